@@ -1,0 +1,1194 @@
+// gradhip engine: device model, paged KV cache, the per-token step (eager,
+// hipGraph-replayed), the on-GPU generate loop, and the C ABI of
+// include/gradhip.h.
+#include "../../include/gradhip.h"
+#include "checkpoint.h"
+#include "kernels_attn.h"
+#include "kernels_common.h"
+#include "kernels_gemm.h"
+#include "kernels_gemv.h"
+#include "kernels_pick.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <numeric>
+#include <string>
+#include <vector>
+
+namespace gh {
+
+// ------------------------------------------------------------------ errors
+
+struct ApiError {
+    gh_status code;
+    std::string msg;
+};
+
+static thread_local std::string g_last_error;
+
+[[noreturn]] static void throw_device(hipError_t e, const char* what, const char* file, int line) {
+    throw ApiError{GH_ERR_DEVICE, std::string("HIP error in ") + what + ": " + hipGetErrorString(e)
+                                      + " (" + file + ":" + std::to_string(line) + ")"};
+}
+
+#define HIP_CHECK(expr)                                                        \
+    do {                                                                       \
+        hipError_t e_ = (expr);                                                \
+        if (e_ != hipSuccess) throw_device(e_, #expr, __FILE__, __LINE__);     \
+    } while (0)
+
+template <typename F>
+static gh_status guard(F&& f) {
+    try {
+        f();
+        return GH_OK;
+    } catch (const ApiError& e) {
+        g_last_error = e.msg;
+        return e.code;
+    } catch (const std::out_of_range& e) {
+        g_last_error = e.what();
+        return GH_ERR_OUT_OF_RANGE;
+    } catch (const std::invalid_argument& e) {
+        g_last_error = e.what();
+        return GH_ERR_INVALID_ARGUMENT;
+    } catch (const std::bad_alloc&) {
+        g_last_error = "out of host memory";
+        return GH_ERR_RUNTIME;
+    } catch (const std::exception& e) {
+        g_last_error = e.what();
+        return GH_ERR_RUNTIME;
+    }
+}
+
+static void require_gpu() {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        throw ApiError{GH_ERR_DEVICE,
+                       "gradhip needs a gfx950 GPU: no HIP device is usable and there is no CPU "
+                       "fallback"};
+    }
+}
+
+// ------------------------------------------------------------ device model
+
+// Layout kernels.  Matrices arrive (in, out) row-major as grad.cpp stores them
+// (inference.cpp:13) and are kept (out, in) so that one output's weights are a
+// contiguous stream.  dst row of source column c is c * row_mul + row_off.
+__global__ void transpose_in_kernel(const float* __restrict__ src, int rows, int cols,
+                                    float* __restrict__ dst, int row_mul, int row_off) {
+    __shared__ float tile[32][33];
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    for (int i = threadIdx.y; i < 32; i += blockDim.y) {
+        const int r = r0 + i, c = c0 + threadIdx.x;
+        if (r < rows && c < cols) tile[i][threadIdx.x] = src[static_cast<size_t>(r) * cols + c];
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 32; i += blockDim.y) {
+        const int c = c0 + i, r = r0 + threadIdx.x;
+        if (r < rows && c < cols)
+            dst[(static_cast<size_t>(c) * row_mul + row_off) * rows + r] = tile[threadIdx.x][i];
+    }
+}
+
+__global__ void transpose_out_kernel(const float* __restrict__ dev, int rows, int cols,
+                                     float* __restrict__ out, int row_mul, int row_off) {
+    __shared__ float tile[32][33];
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    for (int i = threadIdx.y; i < 32; i += blockDim.y) {
+        const int c = c0 + i, r = r0 + threadIdx.x;
+        if (r < rows && c < cols)
+            tile[threadIdx.x][i] = dev[(static_cast<size_t>(c) * row_mul + row_off) * rows + r];
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 32; i += blockDim.y) {
+        const int r = r0 + i, c = c0 + threadIdx.x;
+        if (r < rows && c < cols) out[static_cast<size_t>(r) * cols + c] = tile[i][threadIdx.x];
+    }
+}
+
+struct LayerWeights {
+    float *wqkv, *bqkv;  // (3d, d), 3d
+    float *wo, *bo;      // (d, d), d
+    float *w1, *b1;      // GPT-2: (F, d), F.  Modern: (2F, d) rows (gate_p, up_p) interleaved
+    float *w2, *b2;      // (d, F), d (GPT-2 only)
+    float *g1, *be1, *g2, *be2;
+};
+
+// Where tensor i of the file lives on the device.
+struct Placement {
+    float* dst;
+    bool transpose;
+    int row_mul, row_off;
+};
+
+struct Model {
+    Shape shape;
+    std::optional<Fingerprint> tokenizer;
+    float* blob = nullptr;
+    size_t blob_floats = 0;
+    float* E = nullptr;
+    float* P = nullptr;
+    std::vector<LayerWeights> layers;
+    float *gf = nullptr, *bf = nullptr;
+    float *rope_cos = nullptr, *rope_sin = nullptr;  // (max_len, head_size/2)
+    std::vector<Placement> place;                    // file order
+
+    ~Model() {
+        if (blob) (void)hipFree(blob);
+    }
+};
+
+static size_t align_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
+
+// Carves the weight blob and records where each file tensor goes.
+static void plan_model(Model& m) {
+    const Shape& s = m.shape;
+    const size_t d = s.d_model, F = s.d_ff(), V = s.vocab, C = s.max_len, L = s.layers;
+    size_t off = 0;
+    auto take = [&](size_t n) {
+        const size_t at = off;
+        off = align_up(off + n, 64);  // 256-byte alignment
+        return at;
+    };
+    std::vector<size_t> o;
+    o.push_back(take(V * d));
+    if (!s.modern()) o.push_back(take(C * d));
+    struct LO {
+        size_t wqkv, bqkv, wo, bo, w1, b1, w2, b2, g1, be1, g2, be2;
+    };
+    std::vector<LO> lo(L);
+    for (size_t l = 0; l < L; l++) {
+        lo[l].wqkv = take(3 * d * d);
+        lo[l].bqkv = take(3 * d);
+        lo[l].wo = take(d * d);
+        lo[l].bo = take(d);
+        lo[l].w1 = take((s.modern() ? 2 : 1) * F * d);
+        lo[l].b1 = take(F);
+        lo[l].w2 = take(d * F);
+        lo[l].b2 = take(d);
+        lo[l].g1 = take(d);
+        lo[l].be1 = take(d);
+        lo[l].g2 = take(d);
+        lo[l].be2 = take(d);
+    }
+    const size_t ogf = take(d), obf = take(d);
+    const size_t half = s.head_size() / 2;
+    const size_t ocos = take(C * half + 1), osin = take(C * half + 1);
+    m.blob_floats = off;
+    HIP_CHECK(hipMalloc(&m.blob, off * sizeof(float)));
+    HIP_CHECK(hipMemset(m.blob, 0, off * sizeof(float)));
+
+    float* B = m.blob;
+    m.E = B + o[0];
+    m.P = s.modern() ? nullptr : B + o[1];
+    m.place.push_back({m.E, false, 1, 0});
+    if (!s.modern()) m.place.push_back({m.P, false, 1, 0});
+    m.layers.resize(L);
+    for (size_t l = 0; l < L; l++) {
+        LayerWeights& w = m.layers[l];
+        w = {B + lo[l].wqkv, B + lo[l].bqkv, B + lo[l].wo, B + lo[l].bo, B + lo[l].w1,
+             B + lo[l].b1,   B + lo[l].w2,   B + lo[l].b2, B + lo[l].g1, B + lo[l].be1,
+             B + lo[l].g2,   B + lo[l].be2};
+        for (int q = 0; q < 3; q++) m.place.push_back({w.wqkv + q * d * d, true, 1, 0});
+        m.place.push_back({w.wo, true, 1, 0});
+        for (int q = 0; q < 3; q++) m.place.push_back({w.bqkv + q * d, false, 1, 0});
+        m.place.push_back({w.bo, false, 1, 0});
+        if (s.modern()) {
+            m.place.push_back({w.w1, true, 2, 0});  // gate -> even rows
+            m.place.push_back({w.w1, true, 2, 1});  // up -> odd rows
+            m.place.push_back({w.w2, true, 1, 0});  // down
+        } else {
+            m.place.push_back({w.w1, true, 1, 0});
+            m.place.push_back({w.b1, false, 1, 0});
+            m.place.push_back({w.w2, true, 1, 0});
+            m.place.push_back({w.b2, false, 1, 0});
+        }
+        m.place.push_back({w.g1, false, 1, 0});
+        m.place.push_back({w.be1, false, 1, 0});
+        m.place.push_back({w.g2, false, 1, 0});
+        m.place.push_back({w.be2, false, 1, 0});
+    }
+    m.gf = B + ogf;
+    m.bf = B + obf;
+    m.place.push_back({m.gf, false, 1, 0});
+    m.place.push_back({m.bf, false, 1, 0});
+    m.rope_cos = B + ocos;
+    m.rope_sin = B + osin;
+}
+
+static std::unique_ptr<Model> upload_model(const Shape& shape, const std::vector<const float*>& t,
+                                           const std::optional<Fingerprint>& fp) {
+    require_gpu();
+    auto m = std::make_unique<Model>();
+    m->shape = shape;
+    m->tokenizer = fp;
+    plan_model(*m);
+    const std::vector<TensorSpec> specs = tensor_specs(shape);
+    if (specs.size() != t.size() || specs.size() != m->place.size())
+        throw ApiError{GH_ERR_INVALID_ARGUMENT, "tensor count does not match the model shape"};
+
+    size_t biggest = 0;
+    for (size_t i = 0; i < specs.size(); i++)
+        if (m->place[i].transpose)
+            biggest = std::max(biggest, static_cast<size_t>(specs[i].rows) * specs[i].cols);
+    float* stage = nullptr;
+    HIP_CHECK(hipMalloc(&stage, std::max<size_t>(biggest, 1) * sizeof(float)));
+    try {
+        for (size_t i = 0; i < specs.size(); i++) {
+            const size_t n = static_cast<size_t>(specs[i].rows) * specs[i].cols;
+            const Placement& pl = m->place[i];
+            if (!pl.transpose) {
+                HIP_CHECK(hipMemcpy(pl.dst, t[i], n * sizeof(float), hipMemcpyHostToDevice));
+                continue;
+            }
+            HIP_CHECK(hipMemcpy(stage, t[i], n * sizeof(float), hipMemcpyHostToDevice));
+            const dim3 grid((specs[i].cols + 31) / 32, (specs[i].rows + 31) / 32);
+            transpose_in_kernel<<<grid, dim3(32, 8)>>>(stage, specs[i].rows, specs[i].cols, pl.dst,
+                                                       pl.row_mul, pl.row_off);
+            HIP_CHECK(hipGetLastError());
+            HIP_CHECK(hipDeviceSynchronize());
+        }
+    } catch (...) {
+        (void)hipFree(stage);
+        throw;
+    }
+    HIP_CHECK(hipFree(stage));
+
+    if (shape.modern()) {
+        // The rotation angles of every position, with the reference's own fp32
+        // expression (inference.cpp:169-175).
+        const size_t half = shape.head_size() / 2, C = shape.max_len;
+        std::vector<float> cs(C * half), sn(C * half);
+        for (size_t j = 0; j < half; j++) {
+            const float theta = std::pow(10000.0f, -2.0f * static_cast<float>(j)
+                                                       / static_cast<float>(shape.head_size()));
+            for (size_t pos = 0; pos < C; pos++) {
+                cs[pos * half + j] = std::cos(static_cast<float>(pos) * theta);
+                sn[pos * half + j] = std::sin(static_cast<float>(pos) * theta);
+            }
+        }
+        if (half > 0) {
+            HIP_CHECK(hipMemcpy(m->rope_cos, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
+            HIP_CHECK(hipMemcpy(m->rope_sin, sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
+        }
+    }
+    return m;
+}
+
+// Reads every tensor back in file layout.
+static std::vector<std::vector<float>> download_model(const Model& m) {
+    const std::vector<TensorSpec> specs = tensor_specs(m.shape);
+    size_t biggest = 1;
+    for (const TensorSpec& s : specs) biggest = std::max(biggest, static_cast<size_t>(s.rows) * s.cols);
+    float* stage = nullptr;
+    HIP_CHECK(hipMalloc(&stage, biggest * sizeof(float)));
+    std::vector<std::vector<float>> out;
+    try {
+        for (size_t i = 0; i < specs.size(); i++) {
+            const size_t n = static_cast<size_t>(specs[i].rows) * specs[i].cols;
+            const Placement& pl = m.place[i];
+            std::vector<float> host(n);
+            if (!pl.transpose) {
+                HIP_CHECK(hipMemcpy(host.data(), pl.dst, n * 4, hipMemcpyDeviceToHost));
+            } else {
+                const dim3 grid((specs[i].cols + 31) / 32, (specs[i].rows + 31) / 32);
+                transpose_out_kernel<<<grid, dim3(32, 8)>>>(pl.dst, specs[i].rows, specs[i].cols,
+                                                            stage, pl.row_mul, pl.row_off);
+                HIP_CHECK(hipGetLastError());
+                HIP_CHECK(hipMemcpy(host.data(), stage, n * 4, hipMemcpyDeviceToHost));
+            }
+            out.push_back(std::move(host));
+        }
+    } catch (...) {
+        (void)hipFree(stage);
+        throw;
+    }
+    HIP_CHECK(hipFree(stage));
+    return out;
+}
+
+// ----------------------------------------------------------------- session
+
+struct Session {
+    const Model* m = nullptr;
+    int B = 1;
+    int engine = GH_ENGINE_GRAPH;
+    int page_shift = 6;
+    int pages_per_seq = 0, n_pages = 0;
+    int attn_chunk = 64, attn_max_chunks = 1;
+    int sort_cap = 0;
+    int launches_per_step = 0;
+
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+
+    float* kv_pool = nullptr;
+    int* page_table = nullptr;
+    float *x = nullptr, *h = nullptr, *q = nullptr, *attn = nullptr, *hidden = nullptr,
+          *logits = nullptr;
+    float *work = nullptr, *kept_p = nullptr;
+    int* kept_i = nullptr;
+    float* attn_part = nullptr;
+    unsigned* attn_tickets = nullptr;
+    int* tok = nullptr;   // [B] input ids of the next step
+    int* hist = nullptr;  // [B][hist_stride]
+    int hist_stride = 0;
+    DevState* st = nullptr;
+    int* err = nullptr;
+    float* uniforms = nullptr;  // device copy for generate
+    size_t uniforms_cap = 0;
+    float* logit_log = nullptr;  // per-step logits for gh_session_generate
+    size_t logit_log_cap = 0;
+
+    float* host_logits = nullptr;  // pinned, B * V
+    int* host_ids = nullptr;       // pinned staging for ids
+
+    int pos = 0;     // host mirror of DevState
+    int n_hist = 0;
+    int picks = 0;
+    gh_timing timing{};
+
+    ~Session() {
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (graph) (void)hipGraphDestroy(graph);
+        for (hipEvent_t e : ev)
+            if (e) (void)hipEventDestroy(e);
+        for (void* p : {static_cast<void*>(kv_pool), static_cast<void*>(page_table),
+                        static_cast<void*>(x), static_cast<void*>(h), static_cast<void*>(q),
+                        static_cast<void*>(attn), static_cast<void*>(hidden),
+                        static_cast<void*>(logits), static_cast<void*>(work),
+                        static_cast<void*>(kept_p), static_cast<void*>(kept_i),
+                        static_cast<void*>(attn_part), static_cast<void*>(attn_tickets),
+                        static_cast<void*>(tok), static_cast<void*>(hist), static_cast<void*>(st),
+                        static_cast<void*>(err), static_cast<void*>(uniforms),
+                        static_cast<void*>(logit_log)})
+            if (p) (void)hipFree(p);
+        if (host_logits) (void)hipHostFree(host_logits);
+        if (host_ids) (void)hipHostFree(host_ids);
+        if (stream) (void)hipStreamDestroy(stream);
+    }
+};
+
+static KvLayout kv_layout(const Session& s) {
+    return KvLayout{s.kv_pool,         s.page_table,           s.n_pages, s.pages_per_seq,
+                    s.m->shape.heads,  s.m->shape.head_size(), s.page_shift};
+}
+
+template <typename T>
+static void dev_alloc(T*& p, size_t n) {
+    HIP_CHECK(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(T)));
+    HIP_CHECK(hipMemset(p, 0, std::max<size_t>(n, 1) * sizeof(T)));
+}
+
+// ---- kernel dispatch
+
+template <int PRO, int EPI>
+static void launch_gemv(const GemvParams& p, int batch, hipStream_t st) {
+    const int K = p.K;
+    const bool aligned = (K % 256 == 0) && (p.in_stride % 4 == 0);
+    const int kv = aligned ? K / 256 : 0;
+    auto go = [&](auto kernel, int rows_per_wave) {
+        const int waves = (p.N + rows_per_wave - 1) / rows_per_wave;
+        const dim3 grid((waves + 3) / 4, batch);
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, p);
+    };
+    switch (kv) {
+        case 1: go(gemv_kernel<1, 2, PRO, EPI>, 4); break;
+        case 2: go(gemv_kernel<2, 2, PRO, EPI>, 4); break;
+        case 3: go(gemv_kernel<3, 2, PRO, EPI>, 4); break;
+        case 4: go(gemv_kernel<4, 2, PRO, EPI>, 4); break;
+        case 8: go(gemv_kernel<8, 1, PRO, EPI>, 2); break;
+        case 12: go(gemv_kernel<12, 1, PRO, EPI>, 2); break;
+        default: go(gemv_kernel<0, 1, PRO, EPI>, 2); break;
+    }
+    HIP_CHECK(hipGetLastError());
+}
+
+static void launch_attn(const AttnParams& p, int batch, hipStream_t st) {
+    const int hs = p.kv.head_size;
+    const dim3 grid(p.max_chunks, p.kv.heads, batch);
+    const size_t lds = (static_cast<size_t>(p.chunk) + 4 * hs + 8) * sizeof(float);
+    switch (hs) {
+        case 8: hipLaunchKernelGGL(attn_decode_kernel<8>, grid, dim3(256), lds, st, p); break;
+        case 16: hipLaunchKernelGGL(attn_decode_kernel<16>, grid, dim3(256), lds, st, p); break;
+        case 32: hipLaunchKernelGGL(attn_decode_kernel<32>, grid, dim3(256), lds, st, p); break;
+        case 64: hipLaunchKernelGGL(attn_decode_kernel<64>, grid, dim3(256), lds, st, p); break;
+        case 128: hipLaunchKernelGGL(attn_decode_kernel<128>, grid, dim3(256), lds, st, p); break;
+        default: hipLaunchKernelGGL(attn_decode_kernel<0>, grid, dim3(256), lds, st, p); break;
+    }
+    HIP_CHECK(hipGetLastError());
+}
+
+// One InferenceSession::step for every sequence (inference.cpp:150-258),
+// enqueued on the session stream.  Returns the number of launches.
+static int enqueue_step(Session& s) {
+    const Model& m = *s.m;
+    const Shape& sh = m.shape;
+    const int d = sh.d_model, F = sh.d_ff(), V = sh.vocab, B = s.B;
+    const bool modern = sh.modern();
+    hipStream_t st = s.stream;
+    int launches = 0;
+
+    hipLaunchKernelGGL(embed_kernel, dim3((d + 255) / 256, B), dim3(256), 0, st, m.E, m.P, s.tok,
+                       s.st, s.x, d);
+    HIP_CHECK(hipGetLastError());
+    launches++;
+
+    const bool batched = use_batched_gemm(B);
+    for (int l = 0; l < sh.layers; l++) {
+        const LayerWeights& w = m.layers[l];
+        GemvParams g{};
+        g.kv = kv_layout(s);
+        g.layer = l;
+        g.d_model = d;
+        g.st = s.st;
+
+        // norm1 -> fused Q,K,V projection (+bias, RoPE) -> q buffer / cache row
+        g.W = w.wqkv;
+        g.bias = w.bqkv;
+        g.N = 3 * d;
+        g.K = d;
+        g.in = s.x;
+        g.in_stride = d;
+        g.gamma = w.g1;
+        g.beta = w.be1;
+        g.out = s.q;
+        g.out_stride = d;
+        g.rope = modern;
+        g.rope_cos = m.rope_cos;
+        g.rope_sin = m.rope_sin;
+        if (batched) {
+            launches += launch_norm_gemm(g, modern ? PRO_RMSNORM : PRO_LAYERNORM, EPI_QKV, B, s.h, st);
+        } else {
+            if (modern)
+                launch_gemv<PRO_RMSNORM, EPI_QKV>(g, B, st);
+            else
+                launch_gemv<PRO_LAYERNORM, EPI_QKV>(g, B, st);
+            launches++;
+        }
+
+        AttnParams a{};
+        a.q = s.q;
+        a.out = s.attn;
+        a.kv = g.kv;
+        a.layer = l;
+        a.d_model = d;
+        a.st = s.st;
+        a.chunk = s.attn_chunk;
+        a.max_chunks = s.attn_max_chunks;
+        a.scale = 1.0f / std::sqrt(static_cast<float>(sh.head_size()));
+        a.part = s.attn_part;
+        a.tickets = s.attn_tickets;
+        launch_attn(a, B, st);
+        launches++;
+
+        // x += b_o + attn @ W_o
+        g.W = w.wo;
+        g.bias = w.bo;
+        g.N = d;
+        g.K = d;
+        g.in = s.attn;
+        g.in_stride = d;
+        g.out = s.x;
+        g.out_stride = d;
+        if (batched) {
+            launches += launch_norm_gemm(g, PRO_PLAIN, EPI_RESID, B, s.h, st);
+        } else {
+            launch_gemv<PRO_PLAIN, EPI_RESID>(g, B, st);
+            launches++;
+        }
+
+        // norm2 -> FFN
+        g.in = s.x;
+        g.in_stride = d;
+        g.gamma = w.g2;
+        g.beta = w.be2;
+        g.out = s.hidden;
+        g.out_stride = F;
+        g.W = w.w1;
+        g.K = d;
+        if (modern) {
+            g.bias = nullptr;
+            g.N = 2 * F;
+            if (batched) {
+                launches += launch_norm_gemm(g, PRO_RMSNORM, EPI_SWIGLU, B, s.h, st);
+            } else {
+                launch_gemv<PRO_RMSNORM, EPI_SWIGLU>(g, B, st);
+                launches++;
+            }
+        } else {
+            g.bias = w.b1;
+            g.N = F;
+            if (batched) {
+                launches += launch_norm_gemm(g, PRO_LAYERNORM, EPI_GELU, B, s.h, st);
+            } else {
+                launch_gemv<PRO_LAYERNORM, EPI_GELU>(g, B, st);
+                launches++;
+            }
+        }
+        g.W = w.w2;
+        g.bias = modern ? nullptr : w.b2;
+        g.N = d;
+        g.K = F;
+        g.in = s.hidden;
+        g.in_stride = F;
+        g.out = s.x;
+        g.out_stride = d;
+        if (batched) {
+            launches += launch_norm_gemm(g, PRO_PLAIN, EPI_RESID, B, s.h, st);
+        } else {
+            launch_gemv<PRO_PLAIN, EPI_RESID>(g, B, st);
+            launches++;
+        }
+    }
+
+    // final norm -> logits = h @ E^T (inference.cpp:251-254)
+    GemvParams g{};
+    g.W = m.E;
+    g.bias = nullptr;
+    g.N = V;
+    g.K = d;
+    g.in = s.x;
+    g.in_stride = d;
+    g.gamma = m.gf;
+    g.beta = m.bf;
+    g.out = s.logits;
+    g.out_stride = V;
+    if (batched) {
+        launches += launch_norm_gemm(g, modern ? PRO_RMSNORM : PRO_LAYERNORM, EPI_STORE, B, s.h, st);
+    } else {
+        if (modern)
+            launch_gemv<PRO_RMSNORM, EPI_STORE>(g, B, st);
+        else
+            launch_gemv<PRO_LAYERNORM, EPI_STORE>(g, B, st);
+        launches++;
+    }
+
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, st, s.st);
+    HIP_CHECK(hipGetLastError());
+    launches++;
+    return launches;
+}
+
+static void run_step(Session& s) {
+    if (s.engine == GH_ENGINE_GRAPH) {
+        HIP_CHECK(hipGraphLaunch(s.exec, s.stream));
+    } else {
+        enqueue_step(s);
+    }
+    s.pos++;
+}
+
+static void check_capacity(const Session& s) {
+    // inference.cpp:151-153
+    if (s.pos >= s.m->shape.max_len)
+        throw ApiError{GH_ERR_RUNTIME, "InferenceSession: context exceeds max_len"};
+}
+
+static void check_ids(const Session& s, const int32_t* ids, size_t n) {
+    // inference.cpp:154-156
+    for (size_t i = 0; i < n; i++)
+        if (ids[i] < 0 || ids[i] >= s.m->shape.vocab)
+            throw ApiError{GH_ERR_OUT_OF_RANGE, "InferenceSession: token id out of vocab range"};
+}
+
+__global__ void set_state_kernel(DevState* st, int pos, int n_hist, int picks) {
+    st->pos = pos;
+    st->n_hist = n_hist;
+    st->picks = picks;
+}
+
+// tok[b] = hist[b][t]
+__global__ void load_tok_kernel(const int* hist, int stride, int t, int* tok, int B) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < B) tok[b] = hist[static_cast<size_t>(b) * stride + t];
+}
+
+// hist[b][t] = tok[b]
+__global__ void store_hist_kernel(int* hist, int stride, int t, const int* tok, int B) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < B) hist[static_cast<size_t>(b) * stride + t] = tok[b];
+}
+
+static void reset_session(Session& s) {
+    s.pos = 0;
+    s.n_hist = 0;
+    s.picks = 0;
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, s.stream, s.st, 0, 0, 0);
+    HIP_CHECK(hipGetLastError());
+}
+
+static std::unique_ptr<Session> create_session(const Model& m, const gh_session_opts& o) {
+    require_gpu();
+    if (o.batch < 1) throw ApiError{GH_ERR_INVALID_ARGUMENT, "batch must be at least 1"};
+    auto sp = std::make_unique<Session>();
+    Session& s = *sp;
+    s.m = &m;
+    s.B = o.batch;
+    s.engine = o.engine == GH_ENGINE_AUTO ? GH_ENGINE_GRAPH : o.engine;
+    if (s.engine != GH_ENGINE_GRAPH && s.engine != GH_ENGINE_EAGER)
+        throw ApiError{GH_ERR_INVALID_ARGUMENT, "unknown or unavailable engine"};
+    const Shape& sh = m.shape;
+    const int page_tokens = o.page_tokens > 0 ? o.page_tokens : 64;
+    if (page_tokens & (page_tokens - 1))
+        throw ApiError{GH_ERR_INVALID_ARGUMENT, "page_tokens must be a power of two"};
+    s.page_shift = 0;
+    while ((1 << s.page_shift) < page_tokens) s.page_shift++;
+    s.pages_per_seq = (sh.max_len + page_tokens - 1) / page_tokens;
+    s.n_pages = s.pages_per_seq * s.B;
+
+    const size_t d = sh.d_model, F = sh.d_ff(), V = sh.vocab, B = s.B;
+    HIP_CHECK(hipStreamCreate(&s.stream));
+    for (hipEvent_t& e : s.ev) HIP_CHECK(hipEventCreate(&e));
+
+    // Page table: identity, or a fixed scramble to exercise the indirection.
+    std::vector<int> table(static_cast<size_t>(s.n_pages));
+    std::iota(table.begin(), table.end(), 0);
+    if (o.shuffle_pages) {
+        uint64_t x = 0x9E3779B97F4A7C15ull;
+        for (size_t i = table.size(); i > 1; i--) {
+            x ^= x << 13;
+            x ^= x >> 7;
+            x ^= x << 17;
+            std::swap(table[i - 1], table[x % i]);
+        }
+    }
+    dev_alloc(s.page_table, table.size());
+    HIP_CHECK(hipMemcpy(s.page_table, table.data(), table.size() * sizeof(int),
+                        hipMemcpyHostToDevice));
+    const size_t page_floats = 2ull * sh.heads * page_tokens * sh.head_size();
+    dev_alloc(s.kv_pool, static_cast<size_t>(sh.layers) * s.n_pages * page_floats);
+
+    dev_alloc(s.x, B * d);
+    dev_alloc(s.h, B * std::max(d, F));
+    dev_alloc(s.q, B * d);
+    dev_alloc(s.attn, B * d);
+    dev_alloc(s.hidden, B * F);
+    dev_alloc(s.logits, B * V);
+    dev_alloc(s.work, B * V);
+    dev_alloc(s.kept_p, B * V);
+    dev_alloc(s.kept_i, B * V);
+    dev_alloc(s.tok, B);
+    s.hist_stride = sh.max_len + 2;
+    dev_alloc(s.hist, B * s.hist_stride);
+    dev_alloc(s.st, 1);
+    dev_alloc(s.err, 1);
+    HIP_CHECK(hipHostMalloc(&s.host_logits, B * V * sizeof(float)));
+    HIP_CHECK(hipHostMalloc(&s.host_ids, B * s.hist_stride * sizeof(int)));
+
+    // Attention chunking: enough workgroups to cover the GPU, at most 1024
+    // positions per workgroup (their scores live in LDS).
+    int chunk = 64;
+    while (chunk < 1024 && static_cast<long>(B) * sh.heads * ((sh.max_len + chunk - 1) / chunk) > 2048)
+        chunk *= 2;
+    s.attn_chunk = chunk;
+    s.attn_max_chunks = (sh.max_len + chunk - 1) / chunk;
+    dev_alloc(s.attn_part, B * sh.heads * s.attn_max_chunks * (sh.head_size() + 2));
+    dev_alloc(s.attn_tickets, B * sh.heads);
+
+    // LDS the top-p sort may use: the largest power of two that fits next to
+    // the kernel's static arrays.
+    int dev = 0, lds_bytes = 0;
+    HIP_CHECK(hipGetDevice(&dev));
+    HIP_CHECK(hipDeviceGetAttribute(&lds_bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
+    int cap = 1;
+    while (static_cast<size_t>(cap) * 2 * sizeof(float) + 8192 <= static_cast<size_t>(lds_bytes))
+        cap *= 2;
+    s.sort_cap = cap;
+    if (static_cast<size_t>(cap) * sizeof(float) > 48 * 1024) {
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(pick_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      cap * static_cast<int>(sizeof(float))));
+    }
+
+    reset_session(s);
+    HIP_CHECK(hipStreamSynchronize(s.stream));
+
+    if (s.engine == GH_ENGINE_GRAPH) {
+        HIP_CHECK(hipStreamBeginCapture(s.stream, hipStreamCaptureModeThreadLocal));
+        try {
+            s.launches_per_step = enqueue_step(s);
+        } catch (...) {
+            hipGraph_t g = nullptr;
+            (void)hipStreamEndCapture(s.stream, &g);
+            if (g) (void)hipGraphDestroy(g);
+            throw;
+        }
+        HIP_CHECK(hipStreamEndCapture(s.stream, &s.graph));
+        HIP_CHECK(hipGraphInstantiate(&s.exec, s.graph, nullptr, nullptr, 0));
+    } else {
+        // Count the launches of one step without running it twice: a dry capture.
+        HIP_CHECK(hipStreamBeginCapture(s.stream, hipStreamCaptureModeThreadLocal));
+        hipGraph_t g = nullptr;
+        try {
+            s.launches_per_step = enqueue_step(s);
+        } catch (...) {
+            (void)hipStreamEndCapture(s.stream, &g);
+            if (g) (void)hipGraphDestroy(g);
+            throw;
+        }
+        HIP_CHECK(hipStreamEndCapture(s.stream, &g));
+        if (g) (void)hipGraphDestroy(g);
+    }
+    return sp;
+}
+
+static void launch_pick(Session& s, const gh_sampling& o, const float* dev_uniforms, int u_stride,
+                        uint64_t seed) {
+    PickParams p{};
+    p.logits = s.logits;
+    p.work = s.work;
+    p.kept_p = s.kept_p;
+    p.kept_i = s.kept_i;
+    p.V = s.m->shape.vocab;
+    p.hist = s.hist;
+    p.hist_stride = s.hist_stride;
+    p.n_hist = s.n_hist;
+    p.pick_idx = s.picks;
+    p.tok = s.tok;
+    p.temperature = o.temperature;
+    p.top_k = o.top_k;
+    p.top_p = o.top_p;
+    p.penalty = o.repetition_penalty;
+    p.greedy = o.greedy;
+    p.uniforms = dev_uniforms;
+    p.u_stride = u_stride;
+    p.seed_lo = static_cast<unsigned>(seed & 0xFFFFFFFFu);
+    p.seed_hi = static_cast<unsigned>(seed >> 32);
+    p.sort_cap = s.sort_cap;
+    p.err = s.err;
+    const bool need_sort = !o.greedy && o.top_p < 1.0f;
+    const size_t lds = need_sort ? static_cast<size_t>(s.sort_cap) * sizeof(float) : 0;
+    hipLaunchKernelGGL(pick_kernel, dim3(s.B), dim3(kPickThreads), lds, s.stream, p);
+    HIP_CHECK(hipGetLastError());
+    s.n_hist++;
+    s.picks++;
+}
+
+static void check_sampling(const gh_sampling& o) {
+    if (!o.greedy && !(o.temperature > 0.0f))
+        throw ApiError{GH_ERR_INVALID_ARGUMENT, "temperature must be positive"};
+    if (!(o.repetition_penalty > 0.0f))
+        throw ApiError{GH_ERR_INVALID_ARGUMENT, "repetition_penalty must be positive"};
+}
+
+static void check_pick_error(Session& s) {
+    int e = 0;
+    HIP_CHECK(hipMemcpy(&e, s.err, sizeof(int), hipMemcpyDeviceToHost));
+    if (e) {
+        HIP_CHECK(hipMemset(s.err, 0, sizeof(int)));
+        throw ApiError{GH_ERR_RUNTIME,
+                       "top-p sampling without top-k needs more LDS than this vocabulary allows"};
+    }
+}
+
+}  // namespace gh
+
+// ====================================================================== C ABI
+
+using namespace gh;
+
+struct gh_model {
+    std::unique_ptr<Model> impl;
+};
+struct gh_session {
+    std::unique_ptr<Session> impl;
+};
+
+extern "C" {
+
+const char* gh_last_error(void) { return g_last_error.c_str(); }
+
+static Shape shape_of(const gh_config& c) {
+    Shape s;
+    s.arch = c.arch;
+    s.vocab = c.vocab;
+    s.d_model = c.d_model;
+    s.layers = c.layers;
+    s.heads = c.heads;
+    s.max_len = c.max_len;
+    s.dropout = c.dropout;
+    return s;
+}
+
+static void check_config(const gh_config* cfg) {
+    if (!cfg) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null config"};
+    if (cfg->arch != GH_ARCH_GPT2 && cfg->arch != GH_ARCH_MODERN)
+        throw ApiError{GH_ERR_RUNTIME, "unknown architecture tag " + std::to_string(cfg->arch)};
+    validate_shape(shape_of(*cfg));
+}
+
+gh_status gh_model_load(const char* path, gh_model** out) {
+    return guard([&] {
+        if (!path || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *out = nullptr;
+        HostModel hm = read_checkpoint(path);
+        std::vector<const float*> ptrs;
+        for (const auto& t : hm.tensors) ptrs.push_back(t.data());
+        try {
+            auto m = upload_model(hm.shape, ptrs, hm.tokenizer);
+            *out = new gh_model{std::move(m)};
+        } catch (const ApiError& e) {
+            throw ApiError{e.code, std::string("Failed to load model from ") + path + ": " + e.msg};
+        }
+    });
+}
+
+gh_status gh_model_from_host(const gh_config* cfg, const float* const* tensors, int32_t n_tensors,
+                             gh_model** out) {
+    return guard([&] {
+        if (!tensors || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *out = nullptr;
+        check_config(cfg);
+        const Shape s = shape_of(*cfg);
+        if (static_cast<size_t>(n_tensors) != tensor_specs(s).size())
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "tensor count does not match the model shape"};
+        std::vector<const float*> ptrs(tensors, tensors + n_tensors);
+        for (const float* p : ptrs)
+            if (!p) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null tensor"};
+        std::optional<Fingerprint> fp;
+        if (cfg->has_fingerprint) fp = Fingerprint{cfg->tokenizer_kind, cfg->tokenizer_hash};
+        *out = new gh_model{upload_model(s, ptrs, fp)};
+    });
+}
+
+int32_t gh_config_num_tensors(const gh_config* cfg) {
+    int32_t n = -1;
+    (void)guard([&] {
+        check_config(cfg);
+        n = static_cast<int32_t>(tensor_specs(shape_of(*cfg)).size());
+    });
+    return n;
+}
+
+gh_status gh_config_tensor_shape(const gh_config* cfg, int32_t index, int32_t* rows, int32_t* cols) {
+    return guard([&] {
+        check_config(cfg);
+        const auto specs = tensor_specs(shape_of(*cfg));
+        if (index < 0 || static_cast<size_t>(index) >= specs.size())
+            throw ApiError{GH_ERR_OUT_OF_RANGE, "tensor index out of range"};
+        if (rows) *rows = specs[index].rows;
+        if (cols) *cols = specs[index].cols;
+    });
+}
+
+gh_status gh_model_save(const gh_model* m, const char* path) {
+    return guard([&] {
+        if (!m || !path) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        const auto host = download_model(*m->impl);
+        std::vector<const float*> ptrs;
+        for (const auto& t : host) ptrs.push_back(t.data());
+        std::string why;
+        if (!write_checkpoint(path, m->impl->shape, ptrs, m->impl->tokenizer, why))
+            throw ApiError{GH_ERR_RUNTIME, why};
+    });
+}
+
+void gh_model_free(gh_model* m) { delete m; }
+
+gh_status gh_model_get_config(const gh_model* m, gh_config* out) {
+    return guard([&] {
+        if (!m || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        const Shape& s = m->impl->shape;
+        *out = gh_config{};
+        out->arch = s.arch;
+        out->vocab = s.vocab;
+        out->d_model = s.d_model;
+        out->layers = s.layers;
+        out->heads = s.heads;
+        out->max_len = s.max_len;
+        out->d_ff = s.d_ff();
+        out->dropout = s.dropout;
+        if (m->impl->tokenizer) {
+            out->has_fingerprint = 1;
+            out->tokenizer_kind = m->impl->tokenizer->kind;
+            out->tokenizer_hash = m->impl->tokenizer->hash;
+        }
+    });
+}
+
+gh_status gh_session_create(const gh_model* m, const gh_session_opts* opts, gh_session** out) {
+    return guard([&] {
+        if (!m || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *out = nullptr;
+        gh_session_opts o{};
+        o.batch = 1;
+        if (opts) o = *opts;
+        *out = new gh_session{create_session(*m->impl, o)};
+    });
+}
+
+void gh_session_free(gh_session* s) { delete s; }
+
+gh_status gh_session_reset(gh_session* s) {
+    return guard([&] {
+        if (!s) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null session"};
+        reset_session(*s->impl);
+        HIP_CHECK(hipStreamSynchronize(s->impl->stream));
+    });
+}
+
+gh_status gh_session_step(gh_session* sess, const int32_t* ids, float* logits_host) {
+    return guard([&] {
+        if (!sess || !ids) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        check_capacity(s);
+        check_ids(s, ids, s.B);
+        const size_t V = s.m->shape.vocab;
+        std::memcpy(s.host_ids, ids, s.B * sizeof(int));
+        HIP_CHECK(hipMemcpyAsync(s.tok, s.host_ids, s.B * sizeof(int), hipMemcpyHostToDevice,
+                                 s.stream));
+        // The history feeds the repetition penalty of gh_session_pick.
+        if (s.n_hist < s.hist_stride) {
+            hipLaunchKernelGGL(store_hist_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream,
+                               s.hist, s.hist_stride, s.n_hist, s.tok, s.B);
+            HIP_CHECK(hipGetLastError());
+            s.n_hist++;
+        }
+        run_step(s);
+        HIP_CHECK(hipMemcpyAsync(s.host_logits, s.logits, s.B * V * sizeof(float),
+                                 hipMemcpyDeviceToHost, s.stream));
+        HIP_CHECK(hipStreamSynchronize(s.stream));
+        if (logits_host) std::memcpy(logits_host, s.host_logits, s.B * V * sizeof(float));
+    });
+}
+
+gh_status gh_session_logits(gh_session* s, const float** logits) {
+    return guard([&] {
+        if (!s || !logits) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *logits = s->impl->host_logits;
+    });
+}
+
+gh_status gh_session_prefill(gh_session* sess, const int32_t* ids, int32_t len,
+                             float* last_logits_host) {
+    return guard([&] {
+        if (!sess || !ids) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        if (len < 0) throw ApiError{GH_ERR_INVALID_ARGUMENT, "negative length"};
+        if (len == 0) return;
+        if (s.pos + len > s.m->shape.max_len)
+            throw ApiError{GH_ERR_RUNTIME, "InferenceSession: context exceeds max_len"};
+        check_ids(s, ids, static_cast<size_t>(s.B) * len);
+        const size_t V = s.m->shape.vocab;
+        // Stage the ids into the history, then step through them.
+        for (int b = 0; b < s.B; b++)
+            std::memcpy(s.host_ids + static_cast<size_t>(b) * s.hist_stride,
+                        ids + static_cast<size_t>(b) * len, len * sizeof(int));
+        const int base = s.n_hist;
+        if (base + len > s.hist_stride)
+            throw ApiError{GH_ERR_RUNTIME, "InferenceSession: context exceeds max_len"};
+        for (int b = 0; b < s.B; b++)
+            HIP_CHECK(hipMemcpyAsync(s.hist + static_cast<size_t>(b) * s.hist_stride + base,
+                                     s.host_ids + static_cast<size_t>(b) * s.hist_stride,
+                                     len * sizeof(int), hipMemcpyHostToDevice, s.stream));
+        for (int t = 0; t < len; t++) {
+            hipLaunchKernelGGL(load_tok_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
+                               s.hist_stride, base + t, s.tok, s.B);
+            HIP_CHECK(hipGetLastError());
+            run_step(s);
+        }
+        s.n_hist += len;
+        HIP_CHECK(hipMemcpyAsync(s.host_logits, s.logits, s.B * V * sizeof(float),
+                                 hipMemcpyDeviceToHost, s.stream));
+        HIP_CHECK(hipStreamSynchronize(s.stream));
+        if (last_logits_host) std::memcpy(last_logits_host, s.host_logits, s.B * V * sizeof(float));
+    });
+}
+
+int32_t gh_session_position(const gh_session* s) { return s ? s->impl->pos : -1; }
+int32_t gh_session_capacity(const gh_session* s) { return s ? s->impl->m->shape.max_len : -1; }
+int32_t gh_session_vocab(const gh_session* s) { return s ? s->impl->m->shape.vocab : -1; }
+int32_t gh_session_batch(const gh_session* s) { return s ? s->impl->B : -1; }
+
+gh_status gh_session_read_kv(gh_session* sess, int32_t seq, int32_t layer, int32_t kv, int32_t pos,
+                             float* out_host) {
+    return guard([&] {
+        if (!sess || !out_host) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        const Shape& sh = s.m->shape;
+        if (seq < 0 || seq >= s.B || layer < 0 || layer >= sh.layers || kv < 0 || kv > 1 || pos < 0
+            || pos >= s.pos)
+            throw ApiError{GH_ERR_OUT_OF_RANGE, "cache row out of range"};
+        HIP_CHECK(hipStreamSynchronize(s.stream));
+        std::vector<int> table(static_cast<size_t>(s.n_pages));
+        HIP_CHECK(hipMemcpy(table.data(), s.page_table, table.size() * sizeof(int),
+                            hipMemcpyDeviceToHost));
+        const int hs = sh.head_size();
+        const int page = table[static_cast<size_t>(seq) * s.pages_per_seq + (pos >> s.page_shift)];
+        const int slot = pos & ((1 << s.page_shift) - 1);
+        for (int h = 0; h < sh.heads; h++) {
+            const size_t run = ((static_cast<size_t>(layer) * s.n_pages + page) * 2 + kv) * sh.heads + h;
+            const size_t off = ((run << s.page_shift) + slot) * hs;
+            HIP_CHECK(hipMemcpy(out_host + static_cast<size_t>(h) * hs, s.kv_pool + off,
+                                hs * sizeof(float), hipMemcpyDeviceToHost));
+        }
+    });
+}
+
+gh_status gh_session_pick(gh_session* sess, const gh_sampling* opt, const float* uniforms,
+                          uint64_t seed, int32_t* out_ids) {
+    return guard([&] {
+        if (!sess || !opt) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        check_sampling(*opt);
+        if (s.pos == 0) throw ApiError{GH_ERR_RUNTIME, "no logits yet: step or prefill first"};
+        if (s.n_hist >= s.hist_stride)
+            throw ApiError{GH_ERR_RUNTIME, "token history is full"};
+        const float* du = nullptr;
+        if (uniforms) {
+            if (s.uniforms_cap < static_cast<size_t>(s.B)) {
+                if (s.uniforms) HIP_CHECK(hipFree(s.uniforms));
+                s.uniforms = nullptr;
+                dev_alloc(s.uniforms, s.B);
+                s.uniforms_cap = s.B;
+            }
+            HIP_CHECK(hipMemcpyAsync(s.uniforms, uniforms, s.B * sizeof(float),
+                                     hipMemcpyHostToDevice, s.stream));
+            du = s.uniforms;
+        }
+        // The draw index is folded into the pointer: one uniform per sequence here.
+        const int saved = s.picks;
+        if (du) s.picks = 0;
+        launch_pick(s, *opt, du, 1, seed);
+        if (du) s.picks = saved + 1;
+        HIP_CHECK(hipMemcpyAsync(s.host_ids, s.tok, s.B * sizeof(int), hipMemcpyDeviceToHost,
+                                 s.stream));
+        HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_pick_error(s);
+        if (out_ids) std::memcpy(out_ids, s.host_ids, s.B * sizeof(int));
+    });
+}
+
+gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t prompt_len,
+                              int32_t max_tokens, const gh_sampling* opt, const float* uniforms,
+                              uint64_t seed, int32_t* out_tokens, int32_t* out_len,
+                              float* step_logits_host, int32_t* n_steps) {
+    return guard([&] {
+        if (!sess || !opt || !out_tokens || !out_len)
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        const Shape& sh = s.m->shape;
+        check_sampling(*opt);
+        *out_len = 0;
+        if (n_steps) *n_steps = 0;
+        s.timing = gh_timing{};
+        s.timing.launches_per_step = s.launches_per_step;
+        if (prompt_len <= 0) return;  // text_gen.cpp:40: an empty prompt generates nothing
+        if (!prompts) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null prompts"};
+        if (max_tokens < 0) max_tokens = 0;
+        check_ids(s, prompts, static_cast<size_t>(s.B) * prompt_len);
+        if (prompt_len > sh.max_len)
+            throw ApiError{GH_ERR_RUNTIME, "InferenceSession: context exceeds max_len"};
+        const size_t B = s.B, V = sh.vocab;
+
+        reset_session(s);
+        for (size_t b = 0; b < B; b++)
+            std::memcpy(s.host_ids + b * s.hist_stride, prompts + b * prompt_len,
+                        prompt_len * sizeof(int));
+        HIP_CHECK(hipMemcpyAsync(s.hist, s.host_ids, B * s.hist_stride * sizeof(int),
+                                 hipMemcpyHostToDevice, s.stream));
+        const float* du = nullptr;
+        if (uniforms && !opt->greedy && max_tokens > 0) {
+            const size_t n = B * max_tokens;
+            if (s.uniforms_cap < n) {
+                if (s.uniforms) HIP_CHECK(hipFree(s.uniforms));
+                s.uniforms = nullptr;
+                dev_alloc(s.uniforms, n);
+                s.uniforms_cap = n;
+            }
+            HIP_CHECK(hipMemcpyAsync(s.uniforms, uniforms, n * sizeof(float), hipMemcpyHostToDevice,
+                                     s.stream));
+            du = s.uniforms;
+        }
+        const size_t max_steps = static_cast<size_t>(prompt_len) + max_tokens;
+        if (step_logits_host) {
+            const size_t need = max_steps * B * V;
+            if (s.logit_log_cap < need) {
+                if (s.logit_log) HIP_CHECK(hipFree(s.logit_log));
+                s.logit_log = nullptr;
+                dev_alloc(s.logit_log, need);
+                s.logit_log_cap = need;
+            }
+        }
+        size_t steps = 0;
+        auto log_step = [&] {
+            if (step_logits_host)
+                HIP_CHECK(hipMemcpyAsync(s.logit_log + steps * B * V, s.logits, B * V * sizeof(float),
+                                         hipMemcpyDeviceToDevice, s.stream));
+            steps++;
+        };
+
+        // Prompt: one step per token, logits dropped except the last (text_gen.cpp:44-46).
+        HIP_CHECK(hipEventRecord(s.ev[0], s.stream));
+        for (int t = 0; t < prompt_len; t++) {
+            hipLaunchKernelGGL(load_tok_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
+                               s.hist_stride, t, s.tok, s.B);
+            HIP_CHECK(hipGetLastError());
+            run_step(s);
+            log_step();
+        }
+        s.n_hist = prompt_len;
+        HIP_CHECK(hipEventRecord(s.ev[1], s.stream));
+
+        // Decode (text_gen.cpp:48-64): pick, push, stop at capacity, else step.
+        int decode_steps = 0;
+        for (int i = 0; i < max_tokens; i++) {
+            launch_pick(s, *opt, du, max_tokens, seed);
+            if (s.pos >= sh.max_len) break;
+            run_step(s);
+            log_step();
+            decode_steps++;
+        }
+        HIP_CHECK(hipEventRecord(s.ev[2], s.stream));
+
+        const int total = s.n_hist;
+        HIP_CHECK(hipMemcpyAsync(s.host_ids, s.hist, B * s.hist_stride * sizeof(int),
+                                 hipMemcpyDeviceToHost, s.stream));
+        HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_pick_error(s);
+        const size_t out_stride = static_cast<size_t>(prompt_len) + max_tokens;
+        for (size_t b = 0; b < B; b++)
+            std::memcpy(out_tokens + b * out_stride, s.host_ids + b * s.hist_stride,
+                        total * sizeof(int));
+        *out_len = total;
+        if (step_logits_host)
+            HIP_CHECK(hipMemcpy(step_logits_host, s.logit_log, steps * B * V * sizeof(float),
+                                hipMemcpyDeviceToHost));
+        if (n_steps) *n_steps = static_cast<int32_t>(steps);
+        HIP_CHECK(hipEventElapsedTime(&s.timing.prompt_ms, s.ev[0], s.ev[1]));
+        HIP_CHECK(hipEventElapsedTime(&s.timing.decode_ms, s.ev[1], s.ev[2]));
+        s.timing.prompt_steps = prompt_len;
+        s.timing.decode_steps = decode_steps;
+    });
+}
+
+gh_status gh_session_last_timing(const gh_session* s, gh_timing* out) {
+    return guard([&] {
+        if (!s || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *out = s->impl->timing;
+    });
+}
+
+gh_status gh_device_info(char* name, size_t name_len, int32_t* compute_units, int32_t* is_gfx950) {
+    return guard([&] {
+        require_gpu();
+        int dev = 0;
+        HIP_CHECK(hipGetDevice(&dev));
+        hipDeviceProp_t prop;
+        HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+        if (name && name_len) {
+            std::snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+        }
+        if (compute_units) *compute_units = prop.multiProcessorCount;
+        if (is_gfx950) *is_gfx950 = std::strstr(prop.gcnArchName, "gfx950") != nullptr;
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,214 @@
+// Batch-1 projections: one wavefront per pair of output rows, weights stored
+// (out, in) so each row is one contiguous fp32 stream; the norm that precedes
+// the projection is recomputed per wavefront in registers (no LDS, no block
+// barrier), and the op that follows it (bias, RoPE + cache write, residual add,
+// GELU, SwiGLU) runs in the epilogue.
+//
+// Restates matvec / matvec_add / matvec_nobias / layer_norm_row / rope_row /
+// gelu_row / silu_row of src/transformer/inference.cpp:14-115 as fused kernels.
+#pragma once
+
+#include "kernels_common.h"
+
+namespace gh {
+
+enum Prologue { PRO_PLAIN = 0, PRO_LAYERNORM = 1, PRO_RMSNORM = 2 };
+enum Epilogue { EPI_STORE = 0, EPI_QKV = 1, EPI_RESID = 2, EPI_GELU = 3, EPI_SWIGLU = 4 };
+
+struct GemvParams {
+    const float* W;     // (N, K) row-major: row n holds the weights of output n
+    const float* bias;  // N floats or nullptr
+    int N, K;
+    const float* in;  // [batch][in_stride]
+    int in_stride;
+    const float* gamma;  // norm gain / shift (K floats) for PRO_*NORM
+    const float* beta;
+    float* out;  // [batch][out_stride]
+    int out_stride;
+    // EPI_QKV: rows [0,d) are q, [d,2d) k, [2d,3d) v.
+    KvLayout kv;
+    int layer;
+    int d_model;
+    int rope;               // rotate q and k pairs (2j, 2j+1)
+    const float* rope_cos;  // [max_len][head_size/2]
+    const float* rope_sin;
+    const DevState* st;
+};
+
+// One projected value of the fused QKV product goes to the q buffer or straight
+// into the cache row of the current position (inference.cpp:195-199).
+__device__ __forceinline__ void store_qkv(const GemvParams& p, int b, int row, float v, int pos) {
+    const int d = p.d_model;
+    const int sec = row / d, c = row - sec * d;
+    if (sec == 0) {
+        p.out[static_cast<size_t>(b) * p.out_stride + c] = v;
+    } else {
+        const int hs = p.kv.head_size;
+        const int head = c / hs, j = c - head * hs;
+        p.kv.pool[kv_offset(p.kv, p.layer, b, sec - 1, head, pos) + j] = v;
+    }
+}
+
+template <int EPI>
+__device__ __forceinline__ void gemv_epilogue(const GemvParams& p, int b, int row, float v0,
+                                              float v1, bool has1) {
+    if constexpr (EPI == EPI_STORE) {
+        float* o = p.out + static_cast<size_t>(b) * p.out_stride;
+        o[row] = v0 + (p.bias ? p.bias[row] : 0.0f);
+        if (has1) o[row + 1] = v1 + (p.bias ? p.bias[row + 1] : 0.0f);
+    } else if constexpr (EPI == EPI_RESID) {
+        // y += b, then y += x @ W (inference.cpp:22-28)
+        float* o = p.out + static_cast<size_t>(b) * p.out_stride;
+        o[row] = (o[row] + (p.bias ? p.bias[row] : 0.0f)) + v0;
+        if (has1) o[row + 1] = (o[row + 1] + (p.bias ? p.bias[row + 1] : 0.0f)) + v1;
+    } else if constexpr (EPI == EPI_GELU) {
+        float* o = p.out + static_cast<size_t>(b) * p.out_stride;
+        o[row] = gelu_tanh(v0 + p.bias[row]);
+        if (has1) o[row + 1] = gelu_tanh(v1 + p.bias[row + 1]);
+    } else if constexpr (EPI == EPI_SWIGLU) {
+        // rows (2p, 2p+1) = (gate_p, up_p): hidden_p = up * silu(gate) (inference.cpp:234-239)
+        p.out[static_cast<size_t>(b) * p.out_stride + (row >> 1)] = v1 * silu(v0);
+    } else if constexpr (EPI == EPI_QKV) {
+        const int pos = p.st->pos;
+        float a = v0 + p.bias[row];
+        float c = has1 ? v1 + p.bias[row + 1] : 0.0f;
+        if (p.rope && row < 2 * p.d_model) {
+            // head_size is even under RoPE, so (row, row+1) is one rotation pair.
+            const int hs = p.kv.head_size;
+            const int j = ((row % p.d_model) % hs) >> 1;
+            const float cs = p.rope_cos[pos * (hs >> 1) + j];
+            const float sn = p.rope_sin[pos * (hs >> 1) + j];
+            const float ra = a * cs - c * sn;
+            const float rc = a * sn + c * cs;
+            a = ra;
+            c = rc;
+        }
+        store_qkv(p, b, row, a, pos);
+        if (has1) store_qkv(p, b, row + 1, c, pos);
+    }
+}
+
+// KV: float4 loads per lane per row when K == KV * 256 (fast path); KV == 0 is
+// the any-K path.  PAIRS: row pairs per wavefront.
+template <int KV, int PAIRS, int PRO, int EPI>
+__global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
+    constexpr int R = 2 * PAIRS;
+    const int lane = threadIdx.x & 63;
+    const int wid = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int b = blockIdx.y;
+    const int row0 = wid * R;
+    if (row0 >= p.N) return;
+    const int K = p.K;
+    const float* xin = p.in + static_cast<size_t>(b) * p.in_stride;
+    float acc[R];
+
+    if constexpr (KV > 0) {
+        // Weight loads are issued first: they do not depend on the activations.
+        float4 w[R][KV];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = min(row0 + r, p.N - 1);
+            const float4* wr = reinterpret_cast<const float4*>(p.W + static_cast<size_t>(row) * K);
+#pragma unroll
+            for (int i = 0; i < KV; i++) w[r][i] = wr[i * 64 + lane];
+        }
+        float4 h[KV];
+#pragma unroll
+        for (int i = 0; i < KV; i++) h[i] = reinterpret_cast<const float4*>(xin)[i * 64 + lane];
+
+        if constexpr (PRO == PRO_RMSNORM) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int i = 0; i < KV; i++) ss += dot4(h[i], h[i]);
+            ss = wave_sum(ss);
+            const float r = 1.0f / sqrtf(ss / static_cast<float>(K) + kNormEps);
+#pragma unroll
+            for (int i = 0; i < KV; i++) {
+                const float4 g = reinterpret_cast<const float4*>(p.gamma)[i * 64 + lane];
+                h[i] = make_float4(g.x * h[i].x * r, g.y * h[i].y * r, g.z * h[i].z * r,
+                                   g.w * h[i].w * r);
+            }
+        } else if constexpr (PRO == PRO_LAYERNORM) {
+            float s = 0.0f;
+#pragma unroll
+            for (int i = 0; i < KV; i++) s += (h[i].x + h[i].y) + (h[i].z + h[i].w);
+            const float mean = wave_sum(s) / static_cast<float>(K);
+            float var = 0.0f;
+#pragma unroll
+            for (int i = 0; i < KV; i++) {
+                h[i] = make_float4(h[i].x - mean, h[i].y - mean, h[i].z - mean, h[i].w - mean);
+                var += dot4(h[i], h[i]);
+            }
+            var = wave_sum(var) / static_cast<float>(K);
+            const float inv_std = 1.0f / sqrtf(var + kNormEps);
+#pragma unroll
+            for (int i = 0; i < KV; i++) {
+                const float4 g = reinterpret_cast<const float4*>(p.gamma)[i * 64 + lane];
+                const float4 be = reinterpret_cast<const float4*>(p.beta)[i * 64 + lane];
+                h[i] = make_float4(g.x * h[i].x * inv_std + be.x, g.y * h[i].y * inv_std + be.y,
+                                   g.z * h[i].z * inv_std + be.z, g.w * h[i].w * inv_std + be.w);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float a = 0.0f;
+#pragma unroll
+            for (int i = 0; i < KV; i++) a += dot4(w[r][i], h[i]);
+            acc[r] = wave_sum(a);
+        }
+    } else {
+        // Any K: the norm statistics come from two strided passes over x, the
+        // normalised value is rebuilt on the fly inside the dot products.
+        float mean = 0.0f, scale = 1.0f;
+        if constexpr (PRO == PRO_RMSNORM) {
+            float ss = 0.0f;
+            for (int k = lane; k < K; k += 64) ss += xin[k] * xin[k];
+            scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(K) + kNormEps);
+        } else if constexpr (PRO == PRO_LAYERNORM) {
+            float s = 0.0f;
+            for (int k = lane; k < K; k += 64) s += xin[k];
+            mean = wave_sum(s) / static_cast<float>(K);
+            float var = 0.0f;
+            for (int k = lane; k < K; k += 64) var += (xin[k] - mean) * (xin[k] - mean);
+            scale = 1.0f / sqrtf(wave_sum(var) / static_cast<float>(K) + kNormEps);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = min(row0 + r, p.N - 1);
+            const float* wr = p.W + static_cast<size_t>(row) * K;
+            float a = 0.0f;
+            for (int k = lane; k < K; k += 64) {
+                float hv = xin[k];
+                if constexpr (PRO == PRO_RMSNORM) hv = p.gamma[k] * hv * scale;
+                if constexpr (PRO == PRO_LAYERNORM) hv = p.gamma[k] * (hv - mean) * scale + p.beta[k];
+                a += wr[k] * hv;
+            }
+            acc[r] = wave_sum(a);
+        }
+    }
+
+    if (lane == 0) {
+#pragma unroll
+        for (int q = 0; q < PAIRS; q++) {
+            const int row = row0 + 2 * q;
+            if (row < p.N) gemv_epilogue<EPI>(p, b, row, acc[2 * q], acc[2 * q + 1], row + 1 < p.N);
+        }
+    }
+}
+
+// x[b] = E[token[b]] * 1.0 (+ P[pos]) — inference.cpp:159-182 (the embedding
+// scale is 1.0, token_embedding.h:12).
+__global__ void embed_kernel(const float* __restrict__ E, const float* __restrict__ P,
+                             const int* __restrict__ tok, const DevState* st, float* x, int d) {
+    const int b = blockIdx.y;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= d) return;
+    float v = E[static_cast<size_t>(tok[b]) * d + j];
+    if (P) v += P[static_cast<size_t>(st->pos) * d + j];
+    x[static_cast<size_t>(b) * d + j] = v;
+}
+
+// pos_++ at the end of a step (inference.cpp:256).
+__global__ void advance_kernel(DevState* st) { st->pos += 1; }
+
+}  // namespace gh

@@ -1,0 +1,36 @@
+"""Builds libgradhip.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(PKG, "csrc")
+LIB_DIR = os.path.join(PKG, "lib")
+LIB = os.path.join(LIB_DIR, "libgradhip.so")
+
+# -packed-fp32-ops is switched off on purpose: some packed fp32 forms have given
+# wrong results on this hardware pool.  No fast-math: GELU/SiLU/softmax/RoPE use
+# the precise expf/tanhf.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fno-fast-math", "-Wall", "-Wno-unused-function",
+]
+SOURCES = ["engine.hip", "checkpoint.cpp"]
+
+
+def build(verbose: bool = True) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, "-o", LIB, *[os.path.join(CSRC, s) for s in SOURCES]]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

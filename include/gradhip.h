@@ -1,0 +1,196 @@
+/*
+ * gradhip — MI355X (gfx950) implementation of grad.cpp's KV-cached token loop.
+ *
+ * Plain C ABI: opaque handles, plain pointers and sizes, status codes.  Each
+ * entry point names the grad.cpp interface it stands in for (paths relative to
+ * the grad.cpp source tree).  All arithmetic is fp32; token ids are int32.
+ *
+ * Threading: a model handle is immutable after creation and may be shared by
+ * sessions on different host threads.  A session owns one HIP stream; calls on
+ * one session must be serialised by the caller (grad.cpp's InferenceSession
+ * and TextGen are not thread-safe either).
+ *
+ * There is no CPU fallback: every compute entry point fails with
+ * GH_ERR_DEVICE when no gfx950 device is usable.
+ */
+#ifndef GRADHIP_H
+#define GRADHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct gh_model gh_model;
+typedef struct gh_session gh_session;
+
+/* Status codes.  1..3 name the C++ exception type grad.cpp throws at the same
+ * point (std::runtime_error, std::out_of_range, std::invalid_argument); the
+ * C++ adapter in gradhip.hpp rethrows exactly those. */
+typedef enum gh_status {
+    GH_OK = 0,
+    GH_ERR_RUNTIME = 1,
+    GH_ERR_OUT_OF_RANGE = 2,
+    GH_ERR_INVALID_ARGUMENT = 3,
+    GH_ERR_DEVICE = 4 /* HIP failure or no usable GPU; surfaces as runtime_error */
+} gh_status;
+
+/* Message of the last failure on the calling thread (never NULL). */
+const char* gh_last_error(void);
+
+enum { GH_ARCH_GPT2 = 0, GH_ARCH_MODERN = 1 }; /* GPTArch, gpt_model.h:31 */
+
+/* Hyper-parameters of a checkpoint: the header of GPTModel::save
+ * (gpt_model.cpp:302-314) plus the derived FFN width (feedforward.h:24-28) and
+ * the optional tokenizer fingerprint trailer (gpt_model.cpp:357-363). */
+typedef struct gh_config {
+    int32_t arch;
+    int32_t vocab;
+    int32_t d_model;
+    int32_t layers;
+    int32_t heads;
+    int32_t max_len;
+    int32_t d_ff;
+    float dropout;
+    int32_t has_fingerprint;
+    uint32_t tokenizer_kind; /* 1 = v1 whitespace BPE, 2 = byte-level BPE */
+    uint64_t tokenizer_hash;
+} gh_config;
+
+/* ------------------------------------------------------------------ model */
+
+/* GPTModel::load (gpt_model.cpp:383-525): reads a "GPTM" v1/v2 file with the
+ * same validation order and the same error texts, then uploads the weights.
+ * Unlike the reference it prints nothing on success. */
+gh_status gh_model_load(const char* path, gh_model** out);
+
+/* Builds a model from host tensors in checkpoint order (gpt_model.cpp:318-355):
+ * E; P (GPT-2 only); per layer W_q W_k W_v W_o b_q b_k b_v b_o, then gate up
+ * down (Modern) or W1 b1 W2 b2 (GPT-2), then norm1 gamma beta, norm2 gamma
+ * beta; final gamma beta.  Matrices are (in, out) row-major as grad.cpp stores
+ * them.  cfg->d_ff is ignored (derived).  Stands in for constructing a
+ * GPTModel and assigning its parameters. */
+gh_status gh_model_from_host(const gh_config* cfg, const float* const* tensors, int32_t n_tensors,
+                             gh_model** out);
+
+/* Number of tensors a checkpoint of this shape holds, and the shape of each. */
+int32_t gh_config_num_tensors(const gh_config* cfg);
+gh_status gh_config_tensor_shape(const gh_config* cfg, int32_t index, int32_t* rows, int32_t* cols);
+
+/* GPTModel::save (gpt_model.cpp:292-381): writes a v2 file, bitwise equal to
+ * the file the model was loaded from (weights are read back from the GPU). */
+gh_status gh_model_save(const gh_model* m, const char* path);
+
+void gh_model_free(gh_model* m);
+gh_status gh_model_get_config(const gh_model* m, gh_config* out);
+
+/* ---------------------------------------------------------------- session */
+
+typedef enum gh_engine {
+    GH_ENGINE_AUTO = 0,
+    GH_ENGINE_GRAPH = 1,     /* one kernel per fused op, whole step replayed as a hipGraph */
+    GH_ENGINE_EAGER = 2,     /* same kernels launched one by one (debugging, profiling) */
+    GH_ENGINE_PERSISTENT = 3 /* one cooperative kernel per step; batch 1 only */
+} gh_engine;
+
+typedef struct gh_session_opts {
+    int32_t batch;       /* independent sequences decoded in lock step (>= 1) */
+    int32_t engine;      /* gh_engine */
+    int32_t page_tokens; /* KV-cache page size in positions; 0 = default (64) */
+    int32_t shuffle_pages; /* non-zero: hand out physical pages in a scrambled order */
+} gh_session_opts;
+
+/* InferenceSession::InferenceSession (inference.cpp:121-148): allocates the
+ * paged KV cache (2 * layers * max_len * d_model floats per sequence) and the
+ * per-step scratch, and records the step graph. */
+gh_status gh_session_create(const gh_model* m, const gh_session_opts* opts, gh_session** out);
+void gh_session_free(gh_session* s);
+
+/* Forgets the context: position 0, empty token history. */
+gh_status gh_session_reset(gh_session* s);
+
+/* InferenceSession::step (inference.cpp:150-258) for every sequence of the
+ * batch: appends ids[b] to sequence b and computes the next-token logits.
+ * logits_host, when non-NULL, receives batch * vocab floats.  Errors as the
+ * reference: GH_ERR_RUNTIME "InferenceSession: context exceeds max_len",
+ * GH_ERR_OUT_OF_RANGE "InferenceSession: token id out of vocab range". */
+gh_status gh_session_step(gh_session* s, const int32_t* ids, float* logits_host);
+
+/* Logits of the last step in session-owned pinned host memory, valid until the
+ * next call on the session (the "valid until the next step() call" rule of
+ * inference.h:20-22).  batch * vocab floats. */
+gh_status gh_session_logits(gh_session* s, const float** logits);
+
+/* Feeds `len` tokens per sequence (ids is batch x len, row-major) in one call;
+ * equivalent to `len` step() calls (text_gen.cpp:44-46) whose logits are
+ * dropped except the last.  last_logits_host may be NULL. */
+gh_status gh_session_prefill(gh_session* s, const int32_t* ids, int32_t len,
+                             float* last_logits_host);
+
+int32_t gh_session_position(const gh_session* s); /* inference.h:27 */
+int32_t gh_session_capacity(const gh_session* s); /* inference.h:28 */
+int32_t gh_session_vocab(const gh_session* s);    /* inference.h:29 */
+int32_t gh_session_batch(const gh_session* s);
+
+/* Copies K (kv = 0, after RoPE) or V (kv = 1) row `pos` of `layer` for sequence
+ * `seq` out of the paged cache: d_model floats in the reference's row layout
+ * (inference.cpp:195-196). */
+gh_status gh_session_read_kv(gh_session* s, int32_t seq, int32_t layer, int32_t kv, int32_t pos,
+                             float* out_host);
+
+/* --------------------------------------------------------------- sampling */
+
+/* SamplingOptions (src/cli/common.h:140-147) as TextGen takes them
+ * (text_gen.h:23-37).  greedy != 0 selects generate_greedy's arg-max. */
+typedef struct gh_sampling {
+    float temperature;
+    int32_t top_k; /* 0 = off */
+    float top_p;   /* 1 = off */
+    float repetition_penalty;
+    int32_t greedy;
+} gh_sampling;
+
+/* One pick from the current logits of every sequence, on the GPU:
+ * logits_with_penalty (text_gen.cpp:14-33) over the session's token history,
+ * then arg-max (text_gen.cpp:52-60) or sample_from_logits (text_gen.cpp:135-209).
+ * uniforms: one float per sequence, or NULL to draw Philox4x32-10(seed,
+ * sequence, pick index).  The picked ids are appended to the history and
+ * written to out_ids (batch int32), but NOT stepped. */
+gh_status gh_session_pick(gh_session* s, const gh_sampling* opt, const float* uniforms,
+                          uint64_t seed, int32_t* out_ids);
+
+/* TextGen::generate_greedy / generate_sample (text_gen.cpp:37-91) for `batch`
+ * prompts of equal length, with the token loop kept on the GPU.  prompts is
+ * batch x prompt_len; out_tokens is batch x (prompt_len + max_tokens) and
+ * receives prompt + generated ids; *out_len their count per sequence.
+ * uniforms is batch x max_tokens (draw i of sequence b at [b * max_tokens + i])
+ * or NULL for the on-device Philox stream.  The session is reset first.
+ * step_logits_host, when non-NULL, receives the logits of every step() call
+ * (steps x batch x vocab) and *n_steps their count. */
+gh_status gh_session_generate(gh_session* s, const int32_t* prompts, int32_t prompt_len,
+                              int32_t max_tokens, const gh_sampling* opt, const float* uniforms,
+                              uint64_t seed, int32_t* out_tokens, int32_t* out_len,
+                              float* step_logits_host, int32_t* n_steps);
+
+/* ------------------------------------------------------------ measurement */
+
+/* GPU time of the last gh_session_generate call, from HIP events recorded on
+ * the session's stream: the prompt steps and the decode steps separately. */
+typedef struct gh_timing {
+    float prompt_ms;
+    float decode_ms;
+    int32_t prompt_steps;
+    int32_t decode_steps;
+    int32_t launches_per_step; /* kernel launches (or graph nodes) in one step */
+} gh_timing;
+gh_status gh_session_last_timing(const gh_session* s, gh_timing* out);
+
+/* Device facts for reports: name, compute units, and whether it is gfx950. */
+gh_status gh_device_info(char* name, size_t name_len, int32_t* compute_units, int32_t* is_gfx950);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
