@@ -348,6 +348,7 @@ struct Session {
 
     float* host_logits = nullptr;  // pinned, B * V
     int* host_ids = nullptr;       // pinned staging for ids
+    int* host_err = nullptr;       // pinned landing spot for the device error flag
 
     int pos = 0;     // host mirror of DevState
     int n_hist = 0;
@@ -371,6 +372,7 @@ struct Session {
             if (p) (void)hipFree(p);
         if (host_logits) (void)hipHostFree(host_logits);
         if (host_ids) (void)hipHostFree(host_ids);
+        if (host_err) (void)hipHostFree(host_err);
         if (stream) (void)hipStreamDestroy(stream);
     }
 };
@@ -425,6 +427,31 @@ static void launch_attn(const AttnParams& p, int batch, hipStream_t st) {
     HIP_CHECK(hipGetLastError());
 }
 
+// Batches of this size and up go to the matrix cores.
+constexpr int kMinGemmBatch = 2;
+
+// One projection with its fused prologue / epilogue; returns the launches made.
+template <int PRO, int EPI>
+static int project(Session& s, GemvParams g, hipStream_t st) {
+    const int B = s.B;
+    if (B >= kMinGemmBatch && gemm_shape_ok(g.K, g.in_stride)) {
+        int launches = 1;
+        if (PRO != PRO_PLAIN) {
+            hipLaunchKernelGGL(norm_rows_kernel, dim3((B + 3) / 4), dim3(256), 0, st, g.in, g.gamma,
+                               g.beta, s.h, B, g.K, static_cast<int>(PRO));
+            HIP_CHECK(hipGetLastError());
+            g.in = s.h;
+            g.in_stride = g.K;
+            launches++;
+        }
+        launch_gemm_mfma<EPI>(g, B, st);
+        HIP_CHECK(hipGetLastError());
+        return launches;
+    }
+    launch_gemv<PRO, EPI>(g, B, st);
+    return 1;
+}
+
 // One InferenceSession::step for every sequence (inference.cpp:150-258),
 // enqueued on the session stream.  Returns the number of launches.
 static int enqueue_step(Session& s) {
@@ -440,7 +467,6 @@ static int enqueue_step(Session& s) {
     HIP_CHECK(hipGetLastError());
     launches++;
 
-    const bool batched = use_batched_gemm(B);
     for (int l = 0; l < sh.layers; l++) {
         const LayerWeights& w = m.layers[l];
         GemvParams g{};
@@ -463,15 +489,8 @@ static int enqueue_step(Session& s) {
         g.rope = modern;
         g.rope_cos = m.rope_cos;
         g.rope_sin = m.rope_sin;
-        if (batched) {
-            launches += launch_norm_gemm(g, modern ? PRO_RMSNORM : PRO_LAYERNORM, EPI_QKV, B, s.h, st);
-        } else {
-            if (modern)
-                launch_gemv<PRO_RMSNORM, EPI_QKV>(g, B, st);
-            else
-                launch_gemv<PRO_LAYERNORM, EPI_QKV>(g, B, st);
-            launches++;
-        }
+        launches += modern ? project<PRO_RMSNORM, EPI_QKV>(s, g, st)
+                           : project<PRO_LAYERNORM, EPI_QKV>(s, g, st);
 
         AttnParams a{};
         a.q = s.q;
@@ -497,12 +516,7 @@ static int enqueue_step(Session& s) {
         g.in_stride = d;
         g.out = s.x;
         g.out_stride = d;
-        if (batched) {
-            launches += launch_norm_gemm(g, PRO_PLAIN, EPI_RESID, B, s.h, st);
-        } else {
-            launch_gemv<PRO_PLAIN, EPI_RESID>(g, B, st);
-            launches++;
-        }
+        launches += project<PRO_PLAIN, EPI_RESID>(s, g, st);
 
         // norm2 -> FFN
         g.in = s.x;
@@ -516,21 +530,11 @@ static int enqueue_step(Session& s) {
         if (modern) {
             g.bias = nullptr;
             g.N = 2 * F;
-            if (batched) {
-                launches += launch_norm_gemm(g, PRO_RMSNORM, EPI_SWIGLU, B, s.h, st);
-            } else {
-                launch_gemv<PRO_RMSNORM, EPI_SWIGLU>(g, B, st);
-                launches++;
-            }
+            launches += project<PRO_RMSNORM, EPI_SWIGLU>(s, g, st);
         } else {
             g.bias = w.b1;
             g.N = F;
-            if (batched) {
-                launches += launch_norm_gemm(g, PRO_LAYERNORM, EPI_GELU, B, s.h, st);
-            } else {
-                launch_gemv<PRO_LAYERNORM, EPI_GELU>(g, B, st);
-                launches++;
-            }
+            launches += project<PRO_LAYERNORM, EPI_GELU>(s, g, st);
         }
         g.W = w.w2;
         g.bias = modern ? nullptr : w.b2;
@@ -540,12 +544,7 @@ static int enqueue_step(Session& s) {
         g.in_stride = F;
         g.out = s.x;
         g.out_stride = d;
-        if (batched) {
-            launches += launch_norm_gemm(g, PRO_PLAIN, EPI_RESID, B, s.h, st);
-        } else {
-            launch_gemv<PRO_PLAIN, EPI_RESID>(g, B, st);
-            launches++;
-        }
+        launches += project<PRO_PLAIN, EPI_RESID>(s, g, st);
     }
 
     // final norm -> logits = h @ E^T (inference.cpp:251-254)
@@ -560,15 +559,8 @@ static int enqueue_step(Session& s) {
     g.beta = m.bf;
     g.out = s.logits;
     g.out_stride = V;
-    if (batched) {
-        launches += launch_norm_gemm(g, modern ? PRO_RMSNORM : PRO_LAYERNORM, EPI_STORE, B, s.h, st);
-    } else {
-        if (modern)
-            launch_gemv<PRO_RMSNORM, EPI_STORE>(g, B, st);
-        else
-            launch_gemv<PRO_LAYERNORM, EPI_STORE>(g, B, st);
-        launches++;
-    }
+    launches += modern ? project<PRO_RMSNORM, EPI_STORE>(s, g, st)
+                       : project<PRO_LAYERNORM, EPI_STORE>(s, g, st);
 
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, st, s.st);
     HIP_CHECK(hipGetLastError());
@@ -681,6 +673,7 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     dev_alloc(s.err, 1);
     HIP_CHECK(hipHostMalloc(&s.host_logits, B * V * sizeof(float)));
     HIP_CHECK(hipHostMalloc(&s.host_ids, B * s.hist_stride * sizeof(int)));
+    HIP_CHECK(hipHostMalloc(&s.host_err, sizeof(int)));
 
     // Attention chunking: enough workgroups to cover the GPU, at most 1024
     // positions per workgroup (their scores live in LDS).
@@ -739,8 +732,10 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     return sp;
 }
 
+// commit: the pick becomes part of the token history right away (the generate
+// loop steps it next); otherwise the caller's following step() records it.
 static void launch_pick(Session& s, const gh_sampling& o, const float* dev_uniforms, int u_stride,
-                        uint64_t seed) {
+                        uint64_t seed, bool commit) {
     PickParams p{};
     p.logits = s.logits;
     p.work = s.work;
@@ -767,7 +762,7 @@ static void launch_pick(Session& s, const gh_sampling& o, const float* dev_unifo
     const size_t lds = need_sort ? static_cast<size_t>(s.sort_cap) * sizeof(float) : 0;
     hipLaunchKernelGGL(pick_kernel, dim3(s.B), dim3(kPickThreads), lds, s.stream, p);
     HIP_CHECK(hipGetLastError());
-    s.n_hist++;
+    if (commit) s.n_hist++;
     s.picks++;
 }
 
@@ -779,8 +774,8 @@ static void check_sampling(const gh_sampling& o) {
 }
 
 static void check_pick_error(Session& s) {
-    int e = 0;
-    HIP_CHECK(hipMemcpy(&e, s.err, sizeof(int), hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpy(s.host_err, s.err, sizeof(int), hipMemcpyDeviceToHost));
+    const int e = *s.host_err;
     if (e) {
         HIP_CHECK(hipMemset(s.err, 0, sizeof(int)));
         throw ApiError{GH_ERR_RUNTIME,
@@ -1056,7 +1051,7 @@ gh_status gh_session_pick(gh_session* sess, const gh_sampling* opt, const float*
         // The draw index is folded into the pointer: one uniform per sequence here.
         const int saved = s.picks;
         if (du) s.picks = 0;
-        launch_pick(s, *opt, du, 1, seed);
+        launch_pick(s, *opt, du, 1, seed, false);
         if (du) s.picks = saved + 1;
         HIP_CHECK(hipMemcpyAsync(s.host_ids, s.tok, s.B * sizeof(int), hipMemcpyDeviceToHost,
                                  s.stream));
@@ -1140,7 +1135,7 @@ gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t 
         // Decode (text_gen.cpp:48-64): pick, push, stop at capacity, else step.
         int decode_steps = 0;
         for (int i = 0; i < max_tokens; i++) {
-            launch_pick(s, *opt, du, max_tokens, seed);
+            launch_pick(s, *opt, du, max_tokens, seed, true);
             if (s.pos >= sh.max_len) break;
             run_step(s);
             log_step();

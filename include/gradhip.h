@@ -156,8 +156,9 @@ typedef struct gh_sampling {
  * logits_with_penalty (text_gen.cpp:14-33) over the session's token history,
  * then arg-max (text_gen.cpp:52-60) or sample_from_logits (text_gen.cpp:135-209).
  * uniforms: one float per sequence, or NULL to draw Philox4x32-10(seed,
- * sequence, pick index).  The picked ids are appended to the history and
- * written to out_ids (batch int32), but NOT stepped. */
+ * sequence, pick index).  The picked ids are written to out_ids (batch int32)
+ * but not stepped: the history the penalty looks at is the tokens stepped so
+ * far, so pass the pick (or another id) to gh_session_step next. */
 gh_status gh_session_pick(gh_session* s, const gh_sampling* opt, const float* uniforms,
                           uint64_t seed, int32_t* out_ids);
 
