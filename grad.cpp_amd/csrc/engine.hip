@@ -1061,6 +1061,65 @@ gh_status gh_session_pick(gh_session* sess, const gh_sampling* opt, const float*
     });
 }
 
+gh_status gh_session_decode(gh_session* sess, int32_t max_tokens, const gh_sampling* opt,
+                            const float* uniforms, uint64_t seed, int32_t* out_ids,
+                            int32_t* out_count) {
+    return guard([&] {
+        if (!sess || !opt || !out_count) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        const Shape& sh = s.m->shape;
+        check_sampling(*opt);
+        *out_count = 0;
+        s.timing = gh_timing{};
+        s.timing.launches_per_step = s.launches_per_step;
+        if (max_tokens <= 0) return;
+        if (s.pos == 0) throw ApiError{GH_ERR_RUNTIME, "no logits yet: step or prefill first"};
+        // Picks land in the history at index n_hist = pos; it holds max_len + 2 entries.
+        const size_t B = s.B;
+        const float* du = nullptr;
+        if (uniforms && !opt->greedy) {
+            const size_t n = B * max_tokens;
+            if (s.uniforms_cap < n) {
+                if (s.uniforms) HIP_CHECK(hipFree(s.uniforms));
+                s.uniforms = nullptr;
+                dev_alloc(s.uniforms, n);
+                s.uniforms_cap = n;
+            }
+            HIP_CHECK(hipMemcpyAsync(s.uniforms, uniforms, n * sizeof(float), hipMemcpyHostToDevice,
+                                     s.stream));
+            du = s.uniforms;
+        }
+        const int first = s.n_hist;
+        const int saved_picks = s.picks;
+        if (du) s.picks = 0;  // uniforms are indexed from this call's first pick
+        HIP_CHECK(hipEventRecord(s.ev[1], s.stream));
+        int made = 0, stepped = 0;
+        for (int i = 0; i < max_tokens; i++) {
+            if (s.n_hist >= s.hist_stride) break;
+            launch_pick(s, *opt, du, max_tokens, seed, true);
+            made++;
+            if (s.pos >= sh.max_len) break;  // text_gen.cpp:62
+            run_step(s);
+            stepped++;
+        }
+        HIP_CHECK(hipEventRecord(s.ev[2], s.stream));
+        if (du) s.picks = saved_picks + made;
+        for (size_t b = 0; b < B; b++)
+            HIP_CHECK(hipMemcpyAsync(s.host_ids + b * s.hist_stride,
+                                     s.hist + b * s.hist_stride + first, made * sizeof(int),
+                                     hipMemcpyDeviceToHost, s.stream));
+        HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_pick_error(s);
+        if (out_ids)
+            for (size_t b = 0; b < B; b++)
+                std::memcpy(out_ids + b * max_tokens, s.host_ids + b * s.hist_stride,
+                            made * sizeof(int));
+        *out_count = made;
+        HIP_CHECK(hipEventElapsedTime(&s.timing.decode_ms, s.ev[1], s.ev[2]));
+        s.timing.decode_steps = stepped;
+    });
+}
+
 gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t prompt_len,
                               int32_t max_tokens, const gh_sampling* opt, const float* uniforms,
                               uint64_t seed, int32_t* out_tokens, int32_t* out_len,

@@ -73,6 +73,7 @@ SYMBOLS = {
     "gh_session_batch": (C.c_int32, [_vp]),
     "gh_session_read_kv": (C.c_int, [_vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, _f32p]),
     "gh_session_pick": (C.c_int, [_vp, C.POINTER(GhSampling), _f32p, C.c_uint64, _i32p]),
+    "gh_session_decode": (C.c_int, [_vp, C.c_int32, C.POINTER(GhSampling), _f32p, C.c_uint64, _i32p, _i32p]),
     "gh_session_generate": (C.c_int, [_vp, _i32p, C.c_int32, C.c_int32, C.POINTER(GhSampling), _f32p,
                                       C.c_uint64, _i32p, _i32p, _f32p, _i32p]),
     "gh_session_last_timing": (C.c_int, [_vp, C.POINTER(GhTiming)]),
@@ -235,6 +236,20 @@ class Session:
                                               u.ctypes.data_as(_f32p) if u is not None else None,
                                               seed, out.ctypes.data_as(_i32p)))
         return out
+
+    def decode(self, max_tokens, opt: GhSampling, uniforms=None, seed=0) -> np.ndarray:
+        """Continues from the current context; returns the picks (batch, n)."""
+        out = np.zeros((self.batch, max(max_tokens, 1)), dtype=np.int32)
+        n = C.c_int32()
+        u = None
+        if uniforms is not None:
+            u = np.ascontiguousarray(uniforms, dtype=np.float32).reshape(self.batch, -1)
+            u = np.ascontiguousarray(u[:, :max_tokens])
+            assert u.shape[1] == max_tokens
+        _check(load_library().gh_session_decode(
+            self._h, max_tokens, C.byref(opt), u.ctypes.data_as(_f32p) if u is not None else None, seed,
+            out.ctypes.data_as(_i32p), C.byref(n)))
+        return out[:, :n.value].copy()
 
     def generate(self, prompts, max_tokens, opt: GhSampling, uniforms=None, seed=0, want_logits=False):
         """Returns tokens (batch, n) and, when asked, step logits (steps, batch, vocab)."""

@@ -162,6 +162,17 @@ typedef struct gh_sampling {
 gh_status gh_session_pick(gh_session* s, const gh_sampling* opt, const float* uniforms,
                           uint64_t seed, int32_t* out_ids);
 
+/* The decode loop of TextGen::generate_* (text_gen.cpp:48-64, :80-89) continued
+ * from the session's current context: up to max_tokens rounds of pick, push,
+ * stop at capacity, else step.  out_ids (batch x max_tokens, row stride
+ * max_tokens) receives the picks, *out_count how many were made per sequence.
+ * uniforms is batch x max_tokens or NULL (on-device Philox; the draw index
+ * continues across calls).  This is what a chat turn that keeps its cache
+ * calls after gh_session_prefill. */
+gh_status gh_session_decode(gh_session* s, int32_t max_tokens, const gh_sampling* opt,
+                            const float* uniforms, uint64_t seed, int32_t* out_ids,
+                            int32_t* out_count);
+
 /* TextGen::generate_greedy / generate_sample (text_gen.cpp:37-91) for `batch`
  * prompts of equal length, with the token loop kept on the GPU.  prompts is
  * batch x prompt_len; out_tokens is batch x (prompt_len + max_tokens) and

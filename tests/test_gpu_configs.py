@@ -1,0 +1,123 @@
+"""The named workloads at their full sizes: GPT-2 22M / 70M and the 69M Llama
+block, batch 1 (greedy and sampled), 64-way batched decode, and a 2048-position
+context.  Weights N(0, 0.02) from a seed, prompts uniform from a seed, as the
+configs say; the CPU oracle runs the same thing."""
+import numpy as np
+import pytest
+
+import gradhip as G
+import oracle_lib as O
+from gradhip import synth
+from helpers import assert_logits_close, check_greedy_stream, check_sampled_stream
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4  # per-step logits, relative to the step's largest logit
+
+
+@pytest.fixture(scope="module")
+def blas():
+    return O.blas_init()
+
+
+def _models(name, seed):
+    cfg = synth.PRESETS[name]
+    W = synth.make_weights(cfg, seed)
+    return cfg, W, O.Model.from_tensors(cfg, W), G.Model.from_tensors(cfg, W)
+
+
+@pytest.fixture(scope="module")
+def llama(blas):
+    return _models("c2", 1002)
+
+
+def test_c0_gpt2_small_greedy_80(blas):
+    cfg, W, om, gm = _models("c0", 1000)
+    prompt = synth.uniform_tokens(16, cfg.vocab, 2000)
+    for penalty in (1.0, 1.2):
+        ref, rsl = O.generate_greedy(om, prompt, 80, penalty, want_logits=True)
+        got, gsl = G.Session(gm).generate(prompt, 80, G.sampling(greedy=True, repetition_penalty=penalty),
+                                          want_logits=True)
+        assert len(ref) == 96 and len(rsl) == 96  # 16 + 80 fills the context of 96 exactly
+        check_greedy_stream(got[0], ref, rsl, 16, f"c0 penalty {penalty}")
+        if np.array_equal(got[0], ref):
+            for i in range(96):
+                assert_logits_close(gsl[i, 0], rsl[i], TOL, f"c0 step {i}")
+
+
+def test_c1_gpt2_medium_per_step_logits(blas):
+    cfg, W, om, gm = _models("c1", 1001)
+    prompt = synth.uniform_tokens(32, cfg.vocab, 2001)
+    ref, rsl = O.generate_greedy(om, prompt, 224, 1.0, want_logits=True)
+    # teacher-forced on the oracle's tokens so every one of the 256 steps is compared
+    gs = G.Session(gm)
+    for i, t in enumerate(ref[:256]):
+        assert_logits_close(gs.step([t])[0], rsl[i], TOL, f"c1 step {i}")
+    got = G.Session(gm).generate(prompt, 224, G.sampling(greedy=True, repetition_penalty=1.0))
+    check_greedy_stream(got[0], ref, rsl, 32, "c1")
+
+
+def test_c2_llama_sampled_224(llama):
+    cfg, W, om, gm = llama
+    prompt = synth.uniform_tokens(32, cfg.vocab, 2002)
+    u = synth.uniforms(224, 3002)
+    opts = (0.8, 40, 0.9, 1.1)
+    ref, rsl = O.generate_sample(om, prompt, u, 0.8, 224, 1.1, 40, 0.9, want_logits=True)
+    gs = G.Session(gm)
+    got, gsl = gs.generate(prompt, 224, G.sampling(*opts), uniforms=u, want_logits=True)
+    assert len(ref) == 256
+    check_sampled_stream(got[0], ref, rsl, 32, u, opts, "c2")
+    if np.array_equal(got[0], ref):
+        for i in range(256):
+            assert_logits_close(gsl[i, 0], rsl[i], TOL, f"c2 step {i}")
+    assert np.array_equal(gs.generate(prompt, 224, G.sampling(*opts), seed=3002), got)
+
+
+def test_c3_llama_batch64_greedy(llama):
+    cfg, W, om, gm = llama
+    B = 64
+    prompts = np.stack([synth.uniform_tokens(128, cfg.vocab, 2003, stream=b) for b in range(B)])
+    opt = G.sampling(greedy=True, repetition_penalty=1.0)
+    got = G.Session(gm, batch=B).generate(prompts, 128, opt)
+    assert got.shape == (B, 256)
+    assert np.array_equal(got[:, :128], prompts)
+    # the CPU oracle, run per sequence, on a sample of the batch
+    for b in (0, 17, 63):
+        ref, rsl = O.generate_greedy(om, prompts[b], 128, 1.0, want_logits=True)
+        check_greedy_stream(got[b], ref, rsl, 128, f"c3 seq {b}")
+    # every sequence equals its own batch-1 run on the GPU (batch invariance)
+    single = G.Session(gm)
+    for b in range(0, B, 7):
+        one, sl = single.generate(prompts[b], 128, opt, want_logits=True)
+        check_greedy_stream(got[b], one[0], sl[:, 0], 128, f"c3 seq {b} vs batch 1")
+
+
+def test_c4_llama_context_2048(blas):
+    cfg = synth.PRESETS["c4"]
+    W = synth.make_weights(synth.PRESETS["c2"], 1002)  # RoPE has no table: same tensors, longer context
+    om, gm = O.Model.from_tensors(cfg, W), G.Model.from_tensors(cfg, W)
+    B = 2
+    prompts = np.stack([synth.uniform_tokens(1536, cfg.vocab, 2004, stream=b) for b in range(B)])
+    gs = G.Session(gm, batch=B)
+    last = gs.prefill(prompts)
+    assert gs.position == 1536
+    osess = O.Session(om)
+    for t in prompts[1]:
+        ref = osess.step(t)
+    assert_logits_close(last[1], ref, TOL, "c4 logits after the 1536-token prompt")
+    for layer in (0, 7):
+        for pos in (0, 777, 1535):
+            assert np.abs(gs.read_kv(1, layer, 0, pos) - osess.k_row(layer, pos)).max() < 2e-5
+            assert np.abs(gs.read_kv(1, layer, 1, pos) - osess.v_row(layer, pos)).max() < 2e-5
+    # greedy decode to the end of the 2048 context, teacher-forced on the oracle
+    opt = G.sampling(greedy=True, repetition_penalty=1.0)
+    for i in range(64):
+        nxt_ref = O.argmax_first(ref)
+        nxt = gs.pick(opt)
+        if nxt[1] != nxt_ref:
+            srt = np.sort(ref)
+            assert srt[-1] - srt[-2] <= 4e-6 * np.abs(ref).max(), f"c4 decode token {i}"
+        ids = np.array([nxt[0], nxt_ref], dtype=np.int32)
+        got = gs.step(ids)
+        ref = osess.step(nxt_ref)
+        assert_logits_close(got[1], ref, TOL, f"c4 decode step {i}")
