@@ -321,6 +321,8 @@ struct Session {
     int pages_per_seq = 0, n_pages = 0;
     int attn_chunk = 64, attn_max_chunks = 1;
     int sort_cap = 0;
+    int pick_lds_floats = 0;  // > 0: the LDS-resident pick kernel fits (vocab + sort area)
+    bool pick_global_scratch = false;
     int launches_per_step = 0;
 
     hipStream_t stream = nullptr;
@@ -685,19 +687,30 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     dev_alloc(s.attn_part, B * sh.heads * s.attn_max_chunks * (sh.head_size() + 2));
     dev_alloc(s.attn_tickets, B * sh.heads);
 
-    // LDS the top-p sort may use: the largest power of two that fits next to
-    // the kernel's static arrays.
+    // LDS budget of the pick kernels.  The LDS-resident kernel needs the logits
+    // row plus a power-of-two sort area that can hold it; the fallback kernel
+    // sorts in the largest power of two that fits next to its static arrays.
     int dev = 0, lds_bytes = 0;
     HIP_CHECK(hipGetDevice(&dev));
     HIP_CHECK(hipDeviceGetAttribute(&lds_bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
+    const size_t reserve = 8192;
     int cap = 1;
-    while (static_cast<size_t>(cap) * 2 * sizeof(float) + 8192 <= static_cast<size_t>(lds_bytes))
+    while (static_cast<size_t>(cap) * 2 * sizeof(float) + reserve <= static_cast<size_t>(lds_bytes))
         cap *= 2;
     s.sort_cap = cap;
     if (static_cast<size_t>(cap) * sizeof(float) > 48 * 1024) {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(pick_kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize,
                                       cap * static_cast<int>(sizeof(float))));
+    }
+    size_t v2 = 1024;
+    while (v2 < V) v2 *= 2;
+    s.pick_global_scratch = (o.flags & GH_FLAG_PICK_GLOBAL_SCRATCH) != 0;
+    if (!s.pick_global_scratch && (V + v2) * sizeof(float) + reserve <= static_cast<size_t>(lds_bytes)) {
+        s.pick_lds_floats = static_cast<int>(V + v2);
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(pick_lds_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      s.pick_lds_floats * static_cast<int>(sizeof(float))));
     }
 
     reset_session(s);
@@ -758,9 +771,15 @@ static void launch_pick(Session& s, const gh_sampling& o, const float* dev_unifo
     p.seed_hi = static_cast<unsigned>(seed >> 32);
     p.sort_cap = s.sort_cap;
     p.err = s.err;
-    const bool need_sort = !o.greedy && o.top_p < 1.0f;
-    const size_t lds = need_sort ? static_cast<size_t>(s.sort_cap) * sizeof(float) : 0;
-    hipLaunchKernelGGL(pick_kernel, dim3(s.B), dim3(kPickThreads), lds, s.stream, p);
+    if (s.pick_lds_floats > 0) {
+        p.sort_cap = s.pick_lds_floats - p.V;
+        hipLaunchKernelGGL(pick_lds_kernel, dim3(s.B), dim3(kPickThreads),
+                           static_cast<size_t>(s.pick_lds_floats) * sizeof(float), s.stream, p);
+    } else {
+        const bool need_sort = !o.greedy && o.top_p < 1.0f;
+        const size_t lds = need_sort ? static_cast<size_t>(s.sort_cap) * sizeof(float) : 0;
+        hipLaunchKernelGGL(pick_kernel, dim3(s.B), dim3(kPickThreads), lds, s.stream, p);
+    }
     HIP_CHECK(hipGetLastError());
     if (commit) s.n_hist++;
     s.picks++;

@@ -378,4 +378,337 @@ __global__ __launch_bounds__(kPickThreads) void pick_kernel(const PickParams p) 
     }
 }
 
+// ---------------------------------------------------------------------------
+// LDS-resident variant: the whole logits row lives in LDS, every pass over it is
+// an LDS pass, and the serial parts (sorted running sum, final walk) touch only
+// the survivors.  Used whenever vocab + its sort area fit in LDS; the kernel
+// above is the fallback for larger vocabularies.
+
+// Suffix scan of a 256-bin histogram by one wavefront: finds the bin holding the
+// `want`-th largest key and how many keys are wanted inside it.
+__device__ __forceinline__ void select_bin_wave(const unsigned* hist, int want, unsigned* bcast) {
+    const int lane = threadIdx.x;  // wave 0 only
+    unsigned c[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) c[q] = hist[4 * lane + q];
+    const unsigned mine = (c[0] + c[1]) + (c[2] + c[3]);
+    // above = keys in bins of higher lanes
+    unsigned incl = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned v = __shfl_down(incl, o, kWave);
+        if (lane + o < 64) incl += v;
+    }
+    const unsigned above = incl - mine;
+    if (static_cast<unsigned>(want) > above && static_cast<unsigned>(want) <= above + mine) {
+        unsigned left = static_cast<unsigned>(want) - above;
+        int q = 3;
+        for (; q > 0; q--) {
+            if (c[q] >= left) break;
+            left -= c[q];
+        }
+        bcast[0] = static_cast<unsigned>(4 * lane + q);
+        bcast[1] = left;
+    }
+}
+
+__device__ inline float kth_largest_lds(const float* v, int n, int k, unsigned* hist, unsigned* bcast) {
+    unsigned prefix = 0u, mask = 0u;
+    int remaining = k;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0u;
+        __syncthreads();
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const unsigned key = float_key(v[i]);
+            if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (threadIdx.x < 64) select_bin_wave(hist, remaining, bcast);
+        __syncthreads();
+        prefix |= bcast[0] << shift;
+        mask |= 255u << shift;
+        remaining = static_cast<int>(bcast[1]);
+    }
+    return key_float(prefix);
+}
+
+// Ascending bitonic sort of ints, n2 a power of two.
+__device__ inline void bitonic_asc_int(int* s, int n2) {
+    for (int k = 2; k <= n2; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = threadIdx.x; i < n2; i += blockDim.x) {
+                const int ixj = i ^ j;
+                if (ixj > i) {
+                    const int a = s[i], b = s[ixj];
+                    const bool asc = (i & k) == 0;
+                    if (asc ? (a > b) : (a < b)) {
+                        s[i] = b;
+                        s[ixj] = a;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+__device__ __forceinline__ int block_sum_int(int v, int* scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    int r = 0;
+    for (int w = 0; w < nw; w++) r += scratch[w];
+    return r;
+}
+
+constexpr int kOrderedWalkLimit = 2048;  // survivors sorted by index and walked by one lane
+
+__global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams p) {
+    extern __shared__ float lds[];  // [V] logits -> probabilities, then [sort_cap] sort area
+    __shared__ float red[kPickThreads / 64];
+    __shared__ int redi[kPickThreads / 64];
+    __shared__ unsigned hist256[256];
+    __shared__ unsigned bcast[2];
+    __shared__ int win_tok[kPenaltyWindow];
+    __shared__ float fshare[2];
+    __shared__ int ishare[2];
+
+    const int b = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
+    const int V = p.V;
+    const float* logits = p.logits + static_cast<size_t>(b) * V;
+    float* val = lds;
+    float* srt = lds + V;
+    int* hist = p.hist + static_cast<size_t>(b) * p.hist_stride;
+
+    // ---- logits_with_penalty (text_gen.cpp:14-33)
+    for (int i = tid; i < V; i += nt) val[i] = logits[i];
+    const int window = min(kPenaltyWindow, p.n_hist);
+    if (tid < window) win_tok[tid] = hist[p.n_hist - window + tid];
+    __syncthreads();
+    if (p.penalty != 1.0f && tid < window) {
+        const int id = win_tok[tid];
+        bool first = true;
+        for (int e = 0; e < tid; e++) first = first && (win_tok[e] != id);
+        if (first) {
+            int count = 0;
+            for (int e = tid; e < window; e++) count += (win_tok[e] == id);
+            float v = val[id];
+            for (int c = 0; c < count; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
+            val[id] = v;
+        }
+    }
+    __syncthreads();
+
+    int chosen;
+    if (p.greedy) {
+        float best = -INFINITY;
+        int bi = 0x7FFFFFFF;
+        for (int i = tid; i < V; i += nt) {
+            const float v = val[i];
+            if (v > best) {
+                best = v;
+                bi = i;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, kWave);
+            const int oi = __shfl_xor(bi, o, kWave);
+            if (ov > best || (ov == best && oi < bi)) {
+                best = ov;
+                bi = oi;
+            }
+        }
+        if ((tid & 63) == 0) {
+            red[tid >> 6] = best;
+            redi[tid >> 6] = bi;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < nt / 64; w++) {
+                if (red[w] > best || (red[w] == best && redi[w] < bi)) {
+                    best = red[w];
+                    bi = redi[w];
+                }
+            }
+            ishare[0] = (bi == 0x7FFFFFFF) ? 0 : bi;
+        }
+        __syncthreads();
+        chosen = ishare[0];
+    } else {
+        // ---- sample_from_logits (text_gen.cpp:135-209)
+        const float inv_t = 1.0f / p.temperature;
+        for (int i = tid; i < V; i += nt) val[i] = val[i] * inv_t;
+        __syncthreads();
+        if (p.top_k > 0 && p.top_k < V) {
+            const float thr = kth_largest_lds(val, V, p.top_k, hist256, bcast);
+            for (int i = tid; i < V; i += nt)
+                if (val[i] < thr) val[i] = -1e10f;
+            __syncthreads();
+        }
+        float m = -INFINITY;
+        for (int i = tid; i < V; i += nt) m = fmaxf(m, val[i]);
+        m = block_max(m, red);
+        float sum = 0.0f;
+        for (int i = tid; i < V; i += nt) {
+            const float e = expf(val[i] - m);
+            val[i] = e;
+            sum += e;
+        }
+        sum = block_sum(sum, red);
+        const float inv_sum = 1.0f / sum;
+        int nonzero = 0;
+        for (int i = tid; i < V; i += nt) {
+            const float pr = val[i] * inv_sum;
+            val[i] = pr;
+            nonzero += (pr > 0.0f);
+        }
+        int S = block_sum_int(nonzero, redi);  // entries with p > 0
+
+        if (p.top_p < 1.0f) {
+            float cutoff;
+            if (S > p.sort_cap) {
+                if (tid == 0) *p.err = 1;
+                cutoff = 2.0f;
+            } else {
+                int n2 = 1;
+                while (n2 < S) n2 <<= 1;
+                if (tid == 0) ishare[1] = 0;
+                __syncthreads();
+                for (int i = tid; i < V; i += nt) {
+                    const float v = val[i];
+                    if (v > 0.0f) srt[atomicAdd(&ishare[1], 1)] = v;
+                }
+                for (int i = S + tid; i < n2; i += nt) srt[i] = -1.0f;
+                __syncthreads();
+                bitonic_desc(srt, n2);
+                if (tid == 0) {
+                    float cumulative = 0.0f;
+                    int cutoff_idx = 0;
+                    for (int i = 0; i < S; i++) {
+                        cumulative += srt[i];
+                        if (cumulative >= p.top_p) {
+                            cutoff_idx = i;
+                            break;
+                        }
+                    }
+                    fshare[0] = srt[cutoff_idx];
+                }
+                __syncthreads();
+                cutoff = fshare[0];
+            }
+            int kept = 0;
+            for (int i = tid; i < V; i += nt) {
+                const float v = val[i];
+                if (v < cutoff) val[i] = 0.0f;
+                else kept += (v > 0.0f);
+            }
+            S = block_sum_int(kept, redi);
+        }
+        __syncthreads();
+
+        float u;
+        if (p.uniforms) {
+            u = p.uniforms[static_cast<size_t>(b) * p.u_stride + p.pick_idx];
+        } else {
+            const unsigned w = philox4x32_10(static_cast<unsigned>(p.pick_idx) >> 2,
+                                             static_cast<unsigned>(p.pick_idx) & 3u, p.seed_lo,
+                                             p.seed_hi ^ static_cast<unsigned>(b));
+            u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
+        }
+        const bool renorm = p.top_p < 1.0f;
+
+        if (S <= kOrderedWalkLimit && S <= p.sort_cap) {
+            // Few survivors: list their indices, sort ascending, and let one lane
+            // do the exact index-order sums (text_gen.cpp:178-208).
+            int* idx = reinterpret_cast<int*>(srt);
+            int n2 = 1;
+            while (n2 < S) n2 <<= 1;
+            if (tid == 0) ishare[1] = 0;
+            __syncthreads();
+            for (int i = tid; i < V; i += nt)
+                if (val[i] > 0.0f) idx[atomicAdd(&ishare[1], 1)] = i;
+            for (int i = S + tid; i < n2; i += nt) idx[i] = 0x7FFFFFFF;
+            __syncthreads();
+            bitonic_asc_int(idx, n2);
+            if (tid == 0) {
+                float total = 0.0f;
+                if (renorm)
+                    for (int i = 0; i < S; i++) total += val[idx[i]];
+                const bool divide = renorm && total > 0.0f;
+                int pick = V - 1;
+                if (u <= 0.0f) {
+                    pick = 0;
+                } else {
+                    float cumulative = 0.0f;
+                    for (int i = 0; i < S; i++) {
+                        const float pr = val[idx[i]];
+                        cumulative += divide ? pr / total : pr;
+                        if (u <= cumulative) {
+                            pick = idx[i];
+                            break;
+                        }
+                    }
+                }
+                ishare[0] = pick;
+            }
+        } else {
+            // Many survivors: every thread sums a contiguous run of the row in
+            // index order, one lane walks the run totals, then the crossing run.
+            const int run = (V + nt - 1) / nt;
+            const int lo = min(V, tid * run), hi = min(V, lo + run);
+            float part = 0.0f;
+            for (int i = lo; i < hi; i++) part += val[i];
+            float* parts = srt;  // sort area is free again (nt <= sort_cap whenever this path runs)
+            __syncthreads();
+            parts[tid] = part;
+            __syncthreads();
+            if (tid == 0) {
+                float total = 0.0f;
+                if (renorm)
+                    for (int t = 0; t < nt; t++) total += parts[t];
+                const bool divide = renorm && total > 0.0f;
+                int pick = V - 1;
+                if (u <= 0.0f) {
+                    pick = 0;
+                } else {
+                    float cumulative = 0.0f;
+                    for (int t = 0; t < nt; t++) {
+                        const float next = cumulative + (divide ? parts[t] / total : parts[t]);
+                        if (u <= next) {
+                            const int a = min(V, t * run), e = min(V, a + run);
+                            int last = -1;
+                            bool found = false;
+                            for (int i = a; i < e; i++) {
+                                const float pr = val[i];
+                                if (pr > 0.0f) last = i;
+                                cumulative += divide ? pr / total : pr;
+                                if (u <= cumulative && pr > 0.0f) {
+                                    pick = i;
+                                    found = true;
+                                    break;
+                                }
+                            }
+                            if (!found && last >= 0) pick = last;
+                            break;
+                        }
+                        cumulative = next;
+                    }
+                }
+                ishare[0] = pick;
+            }
+        }
+        __syncthreads();
+        chosen = ishare[0];
+    }
+
+    if (tid == 0) {
+        hist[p.n_hist] = chosen;
+        p.tok[b] = chosen;
+    }
+}
+
 }  // namespace gh

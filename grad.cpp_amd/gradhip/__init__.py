@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(PKG, "lib", "libgradhip.so")
 
 GH_OK, GH_ERR_RUNTIME, GH_ERR_OUT_OF_RANGE, GH_ERR_INVALID_ARGUMENT, GH_ERR_DEVICE = range(5)
 ENGINE_AUTO, ENGINE_GRAPH, ENGINE_EAGER, ENGINE_PERSISTENT = range(4)
+FLAG_PICK_GLOBAL_SCRATCH = 1
 
 
 class DeviceError(RuntimeError):
@@ -37,7 +38,7 @@ class GhConfig(C.Structure):
 
 class GhSessionOpts(C.Structure):
     _fields_ = [("batch", C.c_int32), ("engine", C.c_int32), ("page_tokens", C.c_int32),
-                ("shuffle_pages", C.c_int32)]
+                ("shuffle_pages", C.c_int32), ("flags", C.c_int32)]
 
 
 class GhSampling(C.Structure):
@@ -174,9 +175,10 @@ def sampling(temperature=1.0, top_k=0, top_p=1.0, repetition_penalty=1.2, greedy
 class Session:
     """KV-cached decoder state for `batch` sequences (stands in for grad::InferenceSession)."""
 
-    def __init__(self, model: Model, batch=1, engine=ENGINE_AUTO, page_tokens=0, shuffle_pages=False):
+    def __init__(self, model: Model, batch=1, engine=ENGINE_AUTO, page_tokens=0, shuffle_pages=False,
+                 flags=0):
         self.model = model
-        opts = GhSessionOpts(batch, engine, page_tokens, 1 if shuffle_pages else 0)
+        opts = GhSessionOpts(batch, engine, page_tokens, 1 if shuffle_pages else 0, flags)
         h = _vp()
         _check(load_library().gh_session_create(model._h, C.byref(opts), C.byref(h)))
         self._h = h.value

@@ -100,7 +100,12 @@ typedef struct gh_session_opts {
     int32_t engine;      /* gh_engine */
     int32_t page_tokens; /* KV-cache page size in positions; 0 = default (64) */
     int32_t shuffle_pages; /* non-zero: hand out physical pages in a scrambled order */
+    int32_t flags;         /* GH_FLAG_* */
 } gh_session_opts;
+
+/* Keep the sampler's working row in global memory even when it would fit in
+ * LDS (the path vocabularies above ~16k entries take); for testing that path. */
+enum { GH_FLAG_PICK_GLOBAL_SCRATCH = 1 };
 
 /* InferenceSession::InferenceSession (inference.cpp:121-148): allocates the
  * paged KV cache (2 * layers * max_len * d_model floats per sequence) and the

@@ -41,7 +41,7 @@ def test_header_cites_the_reference_for_every_entry_point():
 def test_struct_layouts_match_the_header():
     import ctypes as C
     assert C.sizeof(G.GhConfig) == 48 and G.GhConfig.tokenizer_hash.offset == 40
-    assert C.sizeof(G.GhSessionOpts) == 16
+    assert C.sizeof(G.GhSessionOpts) == 20
     assert C.sizeof(G.GhSampling) == 20
     assert C.sizeof(G.GhTiming) == 20
 

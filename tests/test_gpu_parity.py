@@ -125,16 +125,17 @@ SAMPLERS = [
 ]
 
 
+@pytest.mark.parametrize("flags", [0, G.FLAG_PICK_GLOBAL_SCRATCH])
 @pytest.mark.parametrize("name", ["ref-sanity-gpt2", "hs64-modern", "d256-modern"])
 @pytest.mark.parametrize("penalty", [1.0, 1.2, 2.5])
-def test_generate_greedy_stream(tiny_models, name, penalty):
+def test_generate_greedy_stream(tiny_models, name, penalty, flags):
     cfg, W, om, gm = tiny_models[name]
     prompt = synth.uniform_tokens(5, cfg.vocab, 12)
     prompt[3] = prompt[1]  # a repeated token inside the penalty window
     for max_tokens in (0, 7, cfg.max_len - 5, cfg.max_len + 20):
         ref, rsl = O.generate_greedy(om, prompt, max_tokens, penalty, want_logits=True)
-        got, gsl = G.Session(gm).generate(prompt, max_tokens, G.sampling(greedy=True, repetition_penalty=penalty),
-                                          want_logits=True)
+        got, gsl = G.Session(gm, flags=flags).generate(
+            prompt, max_tokens, G.sampling(greedy=True, repetition_penalty=penalty), want_logits=True)
         check_greedy_stream(got[0], ref, rsl, len(prompt), f"{name} p{penalty} n{max_tokens}")
         assert got.shape[1] == len(ref) and gsl.shape[0] == len(rsl)  # same number of step() calls
         if np.array_equal(got[0], ref):
@@ -142,16 +143,17 @@ def test_generate_greedy_stream(tiny_models, name, penalty):
                 assert_logits_close(gsl[i, 0], rsl[i], TOL, f"{name} step {i}")
 
 
+@pytest.mark.parametrize("flags", [0, G.FLAG_PICK_GLOBAL_SCRATCH])
 @pytest.mark.parametrize("name", ["ref-metal-gpt2", "hs64-modern", "d256-modern"])
 @pytest.mark.parametrize("opts", SAMPLERS)
-def test_generate_sample_stream_under_shared_draws(tiny_models, name, opts):
+def test_generate_sample_stream_under_shared_draws(tiny_models, name, opts, flags):
     cfg, W, om, gm = tiny_models[name]
     T, k, p, pen = opts
     prompt = synth.uniform_tokens(4, cfg.vocab, 13)
     n = cfg.max_len - 4
     u = synth.uniforms(n, 3000)
     ref, rsl = O.generate_sample(om, prompt, u, T, n, pen, k, p, want_logits=True)
-    s = G.Session(gm)
+    s = G.Session(gm, flags=flags)
     opt = G.sampling(T, k, p, pen)
     got = s.generate(prompt, n, opt, uniforms=u)
     check_sampled_stream(got[0], ref, rsl, len(prompt), u, opts, f"{name} {opts}")
