@@ -7,11 +7,13 @@
 #include "kernels_common.h"
 #include "kernels_gemm.h"
 #include "kernels_gemv.h"
+#include "kernels_persist.h"
 #include "kernels_pick.h"
 
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <numeric>
@@ -136,9 +138,11 @@ struct Model {
     float *gf = nullptr, *bf = nullptr;
     float *rope_cos = nullptr, *rope_sin = nullptr;  // (max_len, head_size/2)
     std::vector<Placement> place;                    // file order
+    LayerPtrs* d_layers = nullptr;                   // the layer table, on the device
 
     ~Model() {
         if (blob) (void)hipFree(blob);
+        if (d_layers) (void)hipFree(d_layers);
     }
 };
 
@@ -258,6 +262,14 @@ static std::unique_ptr<Model> upload_model(const Shape& shape, const std::vector
     }
     HIP_CHECK(hipFree(stage));
 
+    {
+        std::vector<LayerPtrs> table;
+        for (const LayerWeights& w : m->layers)
+            table.push_back({w.wqkv, w.bqkv, w.wo, w.bo, w.w1, w.b1, w.w2, w.b2, w.g1, w.be1, w.g2, w.be2});
+        HIP_CHECK(hipMalloc(&m->d_layers, table.size() * sizeof(LayerPtrs)));
+        HIP_CHECK(hipMemcpy(m->d_layers, table.data(), table.size() * sizeof(LayerPtrs),
+                            hipMemcpyHostToDevice));
+    }
     if (shape.modern()) {
         // The rotation angles of every position, with the reference's own fp32
         // expression (inference.cpp:169-175).
@@ -348,6 +360,16 @@ struct Session {
     float* logit_log = nullptr;  // per-step logits for gh_session_generate
     size_t logit_log_cap = 0;
 
+    // persistent engine
+    Cell* cells = nullptr;  // xa, xb, q, kn, vn, at (d each), hid (F), token (1)
+    PersistCtl* ctl = nullptr;
+    unsigned epoch = 1;         // tag base; grows with every step, never reused
+    unsigned arrive_total = 0;  // logits phases completed so far
+    int persist_grid = 0;
+    unsigned long long* prof = nullptr;  // phase timestamps when GRADHIP_PROF_DUMP is set
+    int prof_cap = 0;
+    size_t persist_lds = 0;
+
     float* host_logits = nullptr;  // pinned, B * V
     int* host_ids = nullptr;       // pinned staging for ids
     int* host_err = nullptr;       // pinned landing spot for the device error flag
@@ -358,6 +380,22 @@ struct Session {
     gh_timing timing{};
 
     ~Session() {
+        if (prof) {
+            // Developer aid: phase-end timestamps of the last persistent launch.
+            std::vector<unsigned long long> host(prof_cap);
+            if (hipMemcpy(host.data(), prof, host.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+                if (std::FILE* f = std::fopen(std::getenv("GRADHIP_PROF_DUMP"), "w")) {
+                    for (size_t i = 0; i < host.size() / 2 && host[i]; i++) std::fprintf(f, "%llu\n", host[i]);
+                    std::fprintf(f, "0\n");
+                    for (size_t i = host.size() - 16; i < host.size() - 8; i++) std::fprintf(f, "%llu\n", host[i]);
+                    std::fprintf(f, "0\n");
+                    for (size_t i = host.size() / 2; i + 3 < host.size() && host[i]; i += 4)
+                        std::fprintf(f, "%llu\n%llu\n%llu\n", host[i + 2], host[i], host[i + 1]);
+                    std::fclose(f);
+                }
+            }
+            (void)hipFree(prof);
+        }
         if (exec) (void)hipGraphExecDestroy(exec);
         if (graph) (void)hipGraphDestroy(graph);
         for (hipEvent_t e : ev)
@@ -370,7 +408,8 @@ struct Session {
                         static_cast<void*>(attn_part), static_cast<void*>(attn_tickets),
                         static_cast<void*>(tok), static_cast<void*>(hist), static_cast<void*>(st),
                         static_cast<void*>(err), static_cast<void*>(uniforms),
-                        static_cast<void*>(logit_log)})
+                        static_cast<void*>(logit_log), static_cast<void*>(cells),
+                        static_cast<void*>(ctl)})
             if (p) (void)hipFree(p);
         if (host_logits) (void)hipHostFree(host_logits);
         if (host_ids) (void)hipHostFree(host_ids);
@@ -570,6 +609,130 @@ static int enqueue_step(Session& s) {
     return launches;
 }
 
+// ---- persistent engine
+
+using PersistKernel = void (*)(const PersistParams);
+
+// The shapes the persistent kernel is built for (head size 64, d_model and FFN
+// width multiples of 256); nullptr for anything else.
+static PersistKernel persist_kernel_for(const Shape& sh) {
+    if (sh.head_size() != 64) return nullptr;
+    const int d = sh.d_model, F = sh.d_ff();
+    if (sh.modern()) {
+        if (d == 768 && F == 2048) return persist_decode_kernel<3, 8, true>;
+        return nullptr;
+    }
+    if (d == 512) return persist_decode_kernel<2, 8, false>;
+    if (d == 768) return persist_decode_kernel<3, 12, false>;
+    if (d == 1024) return persist_decode_kernel<4, 16, false>;
+    return nullptr;
+}
+
+static const char* persist_unavailable(const Session& s, int lds_bytes, int cus) {
+    const Shape& sh = s.m->shape;
+    if (s.B != 1) return "the persistent engine decodes one sequence";
+    if (!persist_kernel_for(sh)) return "the persistent engine has no kernel for this model shape";
+    if (sh.max_len > 512) return "the persistent engine handles contexts up to 512";
+    if (s.pick_lds_floats <= 0) return "the vocabulary does not fit the persistent engine's LDS";
+    if (cus < sh.heads) return "the GPU has fewer compute units than the model has heads";
+    (void)lds_bytes;
+    return nullptr;
+}
+
+// One launch: n_prompt steps fed from the history, then rounds of pick + step.
+static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool start_with_pick,
+                        const gh_sampling* o, const float* dev_uniforms, int u_stride, uint64_t seed,
+                        float* logit_log) {
+    const Model& m = *s.m;
+    const Shape& sh = m.shape;
+    if (n_steps <= 0 && n_picks <= 0) return;
+    PersistParams p{};
+    p.E = m.E;
+    p.P = m.P;
+    p.layers = m.d_layers;
+    p.gf = m.gf;
+    p.bf = m.bf;
+    p.rope_cos = m.rope_cos;
+    p.rope_sin = m.rope_sin;
+    p.d = sh.d_model;
+    p.F = sh.d_ff();
+    p.V = sh.vocab;
+    p.L = sh.layers;
+    p.H = sh.heads;
+    p.kv = kv_layout(s);
+    const size_t d = sh.d_model;
+    p.xa = s.cells;
+    p.xb = s.cells + d;
+    p.q = s.cells + 2 * d;
+    p.kn = s.cells + 3 * d;
+    p.vn = s.cells + 4 * d;
+    p.at = s.cells + 5 * d;
+    p.hid = s.cells + 6 * d;
+    p.tokc = s.cells + 6 * d + sh.d_ff();
+    p.logits = s.logits;
+    p.logit_log = logit_log;
+    p.ctl = s.ctl;
+    p.hist = s.hist;
+    p.pos0 = s.pos;
+    p.n_prompt = n_prompt;
+    p.n_steps = n_steps;
+    p.n_picks = n_picks;
+    p.start_with_pick = start_with_pick ? 1 : 0;
+    p.epoch = s.epoch;
+    p.arrive_base = s.arrive_total;
+    p.spin_limit = 1u << 18;
+    p.prof = s.prof;
+    p.prof_cap = s.prof_cap;
+    PickParams& k = p.pick;
+    k.logits = s.logits;
+    k.V = sh.vocab;
+    k.hist = s.hist;
+    k.hist_stride = s.hist_stride;
+    k.n_hist = s.n_hist + n_prompt;
+    k.pick_idx = s.picks;
+    k.tok = s.tok;
+    if (o) {
+        k.temperature = o->temperature;
+        k.top_k = o->top_k;
+        k.top_p = o->top_p;
+        k.penalty = o->repetition_penalty;
+        k.greedy = o->greedy;
+    }
+    k.uniforms = dev_uniforms;
+    k.u_stride = u_stride;
+    k.seed_lo = static_cast<unsigned>(seed & 0xFFFFFFFFu);
+    k.seed_hi = static_cast<unsigned>(seed >> 32);
+    k.sort_cap = s.pick_lds_floats - sh.vocab;
+    k.err = s.err;
+
+    PersistKernel kernel = persist_kernel_for(sh);
+    hipLaunchKernelGGL(kernel, dim3(s.persist_grid), dim3(kPersistThreads), s.persist_lds, s.stream, p);
+    HIP_CHECK(hipGetLastError());
+
+    // Host mirrors.  Logits are produced by the last prompt step and every later one.
+    int logits_phases = 0;
+    for (int i = 0; i < n_steps; i++)
+        if (i >= n_prompt - 1 || logit_log || i == n_steps - 1) logits_phases++;
+    s.arrive_total += static_cast<unsigned>(logits_phases);
+    s.epoch += static_cast<unsigned>(n_steps) + 1u;
+    s.pos += n_steps;
+    s.n_hist += n_prompt + n_picks;
+    s.picks += n_picks;
+}
+
+// After a synchronisation: did the kernel give up waiting somewhere?
+static void check_persist_abort(Session& s) {
+    if (s.engine != GH_ENGINE_PERSISTENT) return;
+    HIP_CHECK(hipMemcpy(s.host_err, &s.ctl->abort, sizeof(int), hipMemcpyDeviceToHost));
+    if (*s.host_err) {
+        unsigned where = 0;
+        HIP_CHECK(hipMemcpy(s.host_err, &s.ctl->where, sizeof(int), hipMemcpyDeviceToHost));
+        where = static_cast<unsigned>(*s.host_err);
+        throw ApiError{GH_ERR_DEVICE, "persistent decode kernel abandoned a wait (phase tag "
+                                          + std::to_string(where) + "); the session is unusable"};
+    }
+}
+
 static void run_step(Session& s) {
     if (s.engine == GH_ENGINE_GRAPH) {
         HIP_CHECK(hipGraphLaunch(s.exec, s.stream));
@@ -625,9 +788,9 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     Session& s = *sp;
     s.m = &m;
     s.B = o.batch;
-    s.engine = o.engine == GH_ENGINE_AUTO ? GH_ENGINE_GRAPH : o.engine;
-    if (s.engine != GH_ENGINE_GRAPH && s.engine != GH_ENGINE_EAGER)
-        throw ApiError{GH_ERR_INVALID_ARGUMENT, "unknown or unavailable engine"};
+    s.engine = o.engine;
+    if (s.engine < GH_ENGINE_AUTO || s.engine > GH_ENGINE_PERSISTENT)
+        throw ApiError{GH_ERR_INVALID_ARGUMENT, "unknown engine"};
     const Shape& sh = m.shape;
     const int page_tokens = o.page_tokens > 0 ? o.page_tokens : 64;
     if (page_tokens & (page_tokens - 1))
@@ -713,10 +876,35 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
                                       s.pick_lds_floats * static_cast<int>(sizeof(float))));
     }
 
+    {
+        hipDeviceProp_t prop;
+        HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+        const char* why = persist_unavailable(s, lds_bytes, prop.multiProcessorCount);
+        if (s.engine == GH_ENGINE_PERSISTENT && why) throw ApiError{GH_ERR_INVALID_ARGUMENT, why};
+        if (s.engine == GH_ENGINE_AUTO) s.engine = why ? GH_ENGINE_GRAPH : GH_ENGINE_PERSISTENT;
+        if (s.engine == GH_ENGINE_PERSISTENT) {
+            const size_t work = d + std::max(d, F) + 192 + kPersistWaves * 68 + s.pages_per_seq;
+            s.persist_lds = std::max(work, static_cast<size_t>(s.pick_lds_floats)) * sizeof(float);
+            s.persist_grid = std::min(prop.multiProcessorCount, 256);
+            dev_alloc(s.cells, 6 * d + F + 1);
+            dev_alloc(s.ctl, 1);
+            if (std::getenv("GRADHIP_PROF_DUMP")) {
+                s.prof_cap = 1 << 16;
+                dev_alloc(s.prof, s.prof_cap);
+            }
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(persist_kernel_for(sh)),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          static_cast<int>(s.persist_lds)));
+            s.launches_per_step = 1;
+        }
+    }
+
     reset_session(s);
     HIP_CHECK(hipStreamSynchronize(s.stream));
 
-    if (s.engine == GH_ENGINE_GRAPH) {
+    if (s.engine == GH_ENGINE_PERSISTENT) {
+        // nothing to record: one launch runs any number of steps
+    } else if (s.engine == GH_ENGINE_GRAPH) {
         HIP_CHECK(hipStreamBeginCapture(s.stream, hipStreamCaptureModeThreadLocal));
         try {
             s.launches_per_step = enqueue_step(s);
@@ -800,6 +988,83 @@ static void check_pick_error(Session& s) {
         throw ApiError{GH_ERR_RUNTIME,
                        "top-p sampling without top-k needs more LDS than this vocabulary allows"};
     }
+}
+
+// Steps through `len` tokens already staged in the history at n_hist.. (the
+// prompt loop of text_gen.cpp:44-46).  log: per-step logits destination or null.
+static void run_prompt(Session& s, int len, float* log, size_t* steps_logged) {
+    const size_t BV = static_cast<size_t>(s.B) * s.m->shape.vocab;
+    if (s.engine == GH_ENGINE_PERSISTENT) {
+        persist_run(s, len, len, 0, false, nullptr, nullptr, 0, 0,
+                    log ? log + *steps_logged * BV : nullptr);
+        if (steps_logged) *steps_logged += len;
+        return;
+    }
+    const int base = s.n_hist;
+    for (int t = 0; t < len; t++) {
+        hipLaunchKernelGGL(load_tok_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
+                           s.hist_stride, base + t, s.tok, s.B);
+        HIP_CHECK(hipGetLastError());
+        run_step(s);
+        if (log) {
+            HIP_CHECK(hipMemcpyAsync(log + *steps_logged * BV, s.logits, BV * sizeof(float),
+                                     hipMemcpyDeviceToDevice, s.stream));
+        }
+        if (steps_logged) (*steps_logged)++;
+    }
+    s.n_hist += len;
+}
+
+// The decode loop of text_gen.cpp:48-64 from the current context: pick, push,
+// stop at capacity, else step.  Returns {picks made, steps run}.
+static std::pair<int, int> run_decode(Session& s, int max_tokens, const gh_sampling& o,
+                                      const float* du, int u_stride, uint64_t seed, float* log,
+                                      size_t* steps_logged) {
+    const int C = s.m->shape.max_len;
+    const size_t BV = static_cast<size_t>(s.B) * s.m->shape.vocab;
+    if (s.engine == GH_ENGINE_PERSISTENT) {
+        int picks = 0, steps = 0, pos = s.pos, nh = s.n_hist;
+        for (int i = 0; i < max_tokens; i++) {
+            if (nh >= s.hist_stride) break;
+            picks++;
+            nh++;
+            if (pos >= C) break;
+            steps++;
+            pos++;
+        }
+        persist_run(s, 0, steps, picks, true, &o, du, u_stride, seed,
+                    log ? log + *steps_logged * BV : nullptr);
+        if (steps_logged) *steps_logged += steps;
+        return {picks, steps};
+    }
+    int picks = 0, steps = 0;
+    for (int i = 0; i < max_tokens; i++) {
+        if (s.n_hist >= s.hist_stride) break;
+        launch_pick(s, o, du, u_stride, seed, true);
+        picks++;
+        if (s.pos >= C) break;
+        run_step(s);
+        steps++;
+        if (log) {
+            HIP_CHECK(hipMemcpyAsync(log + *steps_logged * BV, s.logits, BV * sizeof(float),
+                                     hipMemcpyDeviceToDevice, s.stream));
+        }
+        if (steps_logged) (*steps_logged)++;
+    }
+    return {picks, steps};
+}
+
+// Copies the caller's uniforms to the device (grown on demand); null for none.
+static const float* stage_uniforms(Session& s, const float* uniforms, size_t n) {
+    if (!uniforms || n == 0) return nullptr;
+    if (s.uniforms_cap < n) {
+        if (s.uniforms) HIP_CHECK(hipFree(s.uniforms));
+        s.uniforms = nullptr;
+        dev_alloc(s.uniforms, n);
+        s.uniforms_cap = n;
+    }
+    HIP_CHECK(hipMemcpyAsync(s.uniforms, uniforms, n * sizeof(float), hipMemcpyHostToDevice, s.stream));
+    return s.uniforms;
 }
 
 }  // namespace gh
@@ -958,17 +1223,20 @@ gh_status gh_session_step(gh_session* sess, const int32_t* ids, float* logits_ho
         std::memcpy(s.host_ids, ids, s.B * sizeof(int));
         HIP_CHECK(hipMemcpyAsync(s.tok, s.host_ids, s.B * sizeof(int), hipMemcpyHostToDevice,
                                  s.stream));
-        // The history feeds the repetition penalty of gh_session_pick.
-        if (s.n_hist < s.hist_stride) {
-            hipLaunchKernelGGL(store_hist_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream,
-                               s.hist, s.hist_stride, s.n_hist, s.tok, s.B);
-            HIP_CHECK(hipGetLastError());
+        // The history (index == position) feeds the repetition penalty of later picks.
+        hipLaunchKernelGGL(store_hist_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
+                           s.hist_stride, s.n_hist, s.tok, s.B);
+        HIP_CHECK(hipGetLastError());
+        if (s.engine == GH_ENGINE_PERSISTENT) {
+            persist_run(s, 1, 1, 0, false, nullptr, nullptr, 0, 0, nullptr);
+        } else {
             s.n_hist++;
+            run_step(s);
         }
-        run_step(s);
         HIP_CHECK(hipMemcpyAsync(s.host_logits, s.logits, s.B * V * sizeof(float),
                                  hipMemcpyDeviceToHost, s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_persist_abort(s);
         if (logits_host) std::memcpy(logits_host, s.host_logits, s.B * V * sizeof(float));
     });
 }
@@ -992,26 +1260,19 @@ gh_status gh_session_prefill(gh_session* sess, const int32_t* ids, int32_t len,
         check_ids(s, ids, static_cast<size_t>(s.B) * len);
         const size_t V = s.m->shape.vocab;
         // Stage the ids into the history, then step through them.
-        for (int b = 0; b < s.B; b++)
+        const int base = s.n_hist;
+        for (int b = 0; b < s.B; b++) {
             std::memcpy(s.host_ids + static_cast<size_t>(b) * s.hist_stride,
                         ids + static_cast<size_t>(b) * len, len * sizeof(int));
-        const int base = s.n_hist;
-        if (base + len > s.hist_stride)
-            throw ApiError{GH_ERR_RUNTIME, "InferenceSession: context exceeds max_len"};
-        for (int b = 0; b < s.B; b++)
             HIP_CHECK(hipMemcpyAsync(s.hist + static_cast<size_t>(b) * s.hist_stride + base,
                                      s.host_ids + static_cast<size_t>(b) * s.hist_stride,
                                      len * sizeof(int), hipMemcpyHostToDevice, s.stream));
-        for (int t = 0; t < len; t++) {
-            hipLaunchKernelGGL(load_tok_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
-                               s.hist_stride, base + t, s.tok, s.B);
-            HIP_CHECK(hipGetLastError());
-            run_step(s);
         }
-        s.n_hist += len;
+        run_prompt(s, len, nullptr, nullptr);
         HIP_CHECK(hipMemcpyAsync(s.host_logits, s.logits, s.B * V * sizeof(float),
                                  hipMemcpyDeviceToHost, s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_persist_abort(s);
         if (last_logits_host) std::memcpy(last_logits_host, s.host_logits, s.B * V * sizeof(float));
     });
 }
@@ -1070,7 +1331,7 @@ gh_status gh_session_pick(gh_session* sess, const gh_sampling* opt, const float*
         // The draw index is folded into the pointer: one uniform per sequence here.
         const int saved = s.picks;
         if (du) s.picks = 0;
-        launch_pick(s, *opt, du, 1, seed, false);
+        launch_pick(s, *opt, du, 1, seed, false);  // the stand-alone pick kernel serves every engine
         if (du) s.picks = saved + 1;
         HIP_CHECK(hipMemcpyAsync(s.host_ids, s.tok, s.B * sizeof(int), hipMemcpyDeviceToHost,
                                  s.stream));
@@ -1086,41 +1347,19 @@ gh_status gh_session_decode(gh_session* sess, int32_t max_tokens, const gh_sampl
     return guard([&] {
         if (!sess || !opt || !out_count) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         Session& s = *sess->impl;
-        const Shape& sh = s.m->shape;
         check_sampling(*opt);
         *out_count = 0;
         s.timing = gh_timing{};
         s.timing.launches_per_step = s.launches_per_step;
         if (max_tokens <= 0) return;
         if (s.pos == 0) throw ApiError{GH_ERR_RUNTIME, "no logits yet: step or prefill first"};
-        // Picks land in the history at index n_hist = pos; it holds max_len + 2 entries.
         const size_t B = s.B;
-        const float* du = nullptr;
-        if (uniforms && !opt->greedy) {
-            const size_t n = B * max_tokens;
-            if (s.uniforms_cap < n) {
-                if (s.uniforms) HIP_CHECK(hipFree(s.uniforms));
-                s.uniforms = nullptr;
-                dev_alloc(s.uniforms, n);
-                s.uniforms_cap = n;
-            }
-            HIP_CHECK(hipMemcpyAsync(s.uniforms, uniforms, n * sizeof(float), hipMemcpyHostToDevice,
-                                     s.stream));
-            du = s.uniforms;
-        }
+        const float* du = opt->greedy ? nullptr : stage_uniforms(s, uniforms, B * max_tokens);
         const int first = s.n_hist;
         const int saved_picks = s.picks;
         if (du) s.picks = 0;  // uniforms are indexed from this call's first pick
         HIP_CHECK(hipEventRecord(s.ev[1], s.stream));
-        int made = 0, stepped = 0;
-        for (int i = 0; i < max_tokens; i++) {
-            if (s.n_hist >= s.hist_stride) break;
-            launch_pick(s, *opt, du, max_tokens, seed, true);
-            made++;
-            if (s.pos >= sh.max_len) break;  // text_gen.cpp:62
-            run_step(s);
-            stepped++;
-        }
+        const auto [made, stepped] = run_decode(s, max_tokens, *opt, du, max_tokens, seed, nullptr, nullptr);
         HIP_CHECK(hipEventRecord(s.ev[2], s.stream));
         if (du) s.picks = saved_picks + made;
         for (size_t b = 0; b < B; b++)
@@ -1128,6 +1367,7 @@ gh_status gh_session_decode(gh_session* sess, int32_t max_tokens, const gh_sampl
                                      s.hist + b * s.hist_stride + first, made * sizeof(int),
                                      hipMemcpyDeviceToHost, s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_persist_abort(s);
         check_pick_error(s);
         if (out_ids)
             for (size_t b = 0; b < B; b++)
@@ -1167,64 +1407,32 @@ gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t 
                         prompt_len * sizeof(int));
         HIP_CHECK(hipMemcpyAsync(s.hist, s.host_ids, B * s.hist_stride * sizeof(int),
                                  hipMemcpyHostToDevice, s.stream));
-        const float* du = nullptr;
-        if (uniforms && !opt->greedy && max_tokens > 0) {
-            const size_t n = B * max_tokens;
-            if (s.uniforms_cap < n) {
-                if (s.uniforms) HIP_CHECK(hipFree(s.uniforms));
-                s.uniforms = nullptr;
-                dev_alloc(s.uniforms, n);
-                s.uniforms_cap = n;
-            }
-            HIP_CHECK(hipMemcpyAsync(s.uniforms, uniforms, n * sizeof(float), hipMemcpyHostToDevice,
-                                     s.stream));
-            du = s.uniforms;
-        }
-        const size_t max_steps = static_cast<size_t>(prompt_len) + max_tokens;
+        const float* du =
+            opt->greedy ? nullptr : stage_uniforms(s, uniforms, B * static_cast<size_t>(max_tokens));
+        float* log = nullptr;
         if (step_logits_host) {
-            const size_t need = max_steps * B * V;
+            const size_t need = (static_cast<size_t>(prompt_len) + max_tokens) * B * V;
             if (s.logit_log_cap < need) {
                 if (s.logit_log) HIP_CHECK(hipFree(s.logit_log));
                 s.logit_log = nullptr;
                 dev_alloc(s.logit_log, need);
                 s.logit_log_cap = need;
             }
+            log = s.logit_log;
         }
         size_t steps = 0;
-        auto log_step = [&] {
-            if (step_logits_host)
-                HIP_CHECK(hipMemcpyAsync(s.logit_log + steps * B * V, s.logits, B * V * sizeof(float),
-                                         hipMemcpyDeviceToDevice, s.stream));
-            steps++;
-        };
-
-        // Prompt: one step per token, logits dropped except the last (text_gen.cpp:44-46).
         HIP_CHECK(hipEventRecord(s.ev[0], s.stream));
-        for (int t = 0; t < prompt_len; t++) {
-            hipLaunchKernelGGL(load_tok_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
-                               s.hist_stride, t, s.tok, s.B);
-            HIP_CHECK(hipGetLastError());
-            run_step(s);
-            log_step();
-        }
-        s.n_hist = prompt_len;
+        run_prompt(s, prompt_len, log, &steps);
         HIP_CHECK(hipEventRecord(s.ev[1], s.stream));
-
-        // Decode (text_gen.cpp:48-64): pick, push, stop at capacity, else step.
-        int decode_steps = 0;
-        for (int i = 0; i < max_tokens; i++) {
-            launch_pick(s, *opt, du, max_tokens, seed, true);
-            if (s.pos >= sh.max_len) break;
-            run_step(s);
-            log_step();
-            decode_steps++;
-        }
+        const auto [made, stepped] = run_decode(s, max_tokens, *opt, du, max_tokens, seed, log, &steps);
+        (void)made;
         HIP_CHECK(hipEventRecord(s.ev[2], s.stream));
 
         const int total = s.n_hist;
         HIP_CHECK(hipMemcpyAsync(s.host_ids, s.hist, B * s.hist_stride * sizeof(int),
                                  hipMemcpyDeviceToHost, s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_persist_abort(s);
         check_pick_error(s);
         const size_t out_stride = static_cast<size_t>(prompt_len) + max_tokens;
         for (size_t b = 0; b < B; b++)
@@ -1238,7 +1446,7 @@ gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t 
         HIP_CHECK(hipEventElapsedTime(&s.timing.prompt_ms, s.ev[0], s.ev[1]));
         HIP_CHECK(hipEventElapsedTime(&s.timing.decode_ms, s.ev[1], s.ev[2]));
         s.timing.prompt_steps = prompt_len;
-        s.timing.decode_steps = decode_steps;
+        s.timing.decode_steps = stepped;
     });
 }
 

@@ -43,16 +43,49 @@ __device__ __forceinline__ size_t kv_offset(const KvLayout& kv, int layer, int s
     return ((run << kv.page_shift) + slot) * kv.head_size;
 }
 
+// Device-scope ("sc1") vector loads through a buffer descriptor.  They see data
+// other workgroups of a running kernel wrote with device-scope stores, like an
+// atomic load does, but several can be in flight at once.  Reads past the end
+// of the buffer return zero.
+typedef int v4i __attribute__((ext_vector_type(4)));
+constexpr int kAuxDeviceScope = 16;  // sc1 on gfx94x / gfx950 buffer instructions
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+__device__ __forceinline__ v4i coherent_load16(__amdgpu_buffer_rsrc_t rs, unsigned byte_offset) {
+    return __builtin_amdgcn_raw_buffer_load_b128(rs, byte_offset, 0, kAuxDeviceScope);
+}
+
+// Wavefront reductions on the data-parallel-primitive (DPP) path: lane
+// permutations inside the ALU instead of trips through the LDS crossbar.
+// Four steps fold each row of 16 lanes, two row broadcasts fold the four rows
+// into lane 63, and a scalar read hands the result to every lane.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v, float fill) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), CTRL,
+                                                      ROW_MASK, 0xF, false));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-    return v;
+    v += dpp_move<0xB1, 0xF>(v, 0.0f);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xF>(v, 0.0f);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xF>(v, 0.0f);  // row_half_mirror
+    v += dpp_move<0x140, 0xF>(v, 0.0f);  // row_mirror
+    v += dpp_move<0x142, 0xA>(v, 0.0f);  // row_bcast:15 into rows 1 and 3
+    v += dpp_move<0x143, 0xC>(v, 0.0f);  // row_bcast:31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-    return v;
+    v = fmaxf(v, dpp_move<0xB1, 0xF>(v, v));
+    v = fmaxf(v, dpp_move<0x4E, 0xF>(v, v));
+    v = fmaxf(v, dpp_move<0x141, 0xF>(v, v));
+    v = fmaxf(v, dpp_move<0x140, 0xF>(v, v));
+    v = fmaxf(v, dpp_move<0x142, 0xA>(v, v));
+    v = fmaxf(v, dpp_move<0x143, 0xC>(v, v));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // Block-wide reductions through a small LDS scratch (one float per wave).

@@ -88,6 +88,46 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, int b, int ro
     }
 }
 
+// Normalises a register-resident row slice in place (layer_norm_row,
+// inference.cpp:30-58): lane holds float4 i at elements (i*64 + lane)*4 .. +3 of
+// a K-long row, K = KV * 256.  The two reductions are wave-wide.
+template <int KV, int PRO>
+__device__ __forceinline__ void norm_in_registers(float4 (&h)[KV], const float* gamma,
+                                                  const float* beta, int K, int lane) {
+    if constexpr (PRO == PRO_RMSNORM) {
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < KV; i++) ss += dot4(h[i], h[i]);
+        ss = wave_sum(ss);
+        const float r = 1.0f / sqrtf(ss / static_cast<float>(K) + kNormEps);
+#pragma unroll
+        for (int i = 0; i < KV; i++) {
+            const float4 g = reinterpret_cast<const float4*>(gamma)[i * 64 + lane];
+            h[i] = make_float4(g.x * h[i].x * r, g.y * h[i].y * r, g.z * h[i].z * r, g.w * h[i].w * r);
+        }
+    } else if constexpr (PRO == PRO_LAYERNORM) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < KV; i++) s += (h[i].x + h[i].y) + (h[i].z + h[i].w);
+        const float mean = wave_sum(s) / static_cast<float>(K);
+        float var = 0.0f;
+#pragma unroll
+        for (int i = 0; i < KV; i++) {
+            h[i] = make_float4(h[i].x - mean, h[i].y - mean, h[i].z - mean, h[i].w - mean);
+            var += dot4(h[i], h[i]);
+        }
+        var = wave_sum(var) / static_cast<float>(K);
+        const float inv_std = 1.0f / sqrtf(var + kNormEps);
+#pragma unroll
+        for (int i = 0; i < KV; i++) {
+            const float4 g = reinterpret_cast<const float4*>(gamma)[i * 64 + lane];
+            const float4 be = reinterpret_cast<const float4*>(beta)[i * 64 + lane];
+            h[i] = make_float4(g.x * h[i].x * inv_std + be.x, g.y * h[i].y * inv_std + be.y,
+                               g.z * h[i].z * inv_std + be.z, g.w * h[i].w * inv_std + be.w);
+        }
+    }
+}
+
 // KV: float4 loads per lane per row when K == KV * 256 (fast path); KV == 0 is
 // the any-K path.  PAIRS: row pairs per wavefront.
 template <int KV, int PAIRS, int PRO, int EPI>
@@ -116,39 +156,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
 #pragma unroll
         for (int i = 0; i < KV; i++) h[i] = reinterpret_cast<const float4*>(xin)[i * 64 + lane];
 
-        if constexpr (PRO == PRO_RMSNORM) {
-            float ss = 0.0f;
-#pragma unroll
-            for (int i = 0; i < KV; i++) ss += dot4(h[i], h[i]);
-            ss = wave_sum(ss);
-            const float r = 1.0f / sqrtf(ss / static_cast<float>(K) + kNormEps);
-#pragma unroll
-            for (int i = 0; i < KV; i++) {
-                const float4 g = reinterpret_cast<const float4*>(p.gamma)[i * 64 + lane];
-                h[i] = make_float4(g.x * h[i].x * r, g.y * h[i].y * r, g.z * h[i].z * r,
-                                   g.w * h[i].w * r);
-            }
-        } else if constexpr (PRO == PRO_LAYERNORM) {
-            float s = 0.0f;
-#pragma unroll
-            for (int i = 0; i < KV; i++) s += (h[i].x + h[i].y) + (h[i].z + h[i].w);
-            const float mean = wave_sum(s) / static_cast<float>(K);
-            float var = 0.0f;
-#pragma unroll
-            for (int i = 0; i < KV; i++) {
-                h[i] = make_float4(h[i].x - mean, h[i].y - mean, h[i].z - mean, h[i].w - mean);
-                var += dot4(h[i], h[i]);
-            }
-            var = wave_sum(var) / static_cast<float>(K);
-            const float inv_std = 1.0f / sqrtf(var + kNormEps);
-#pragma unroll
-            for (int i = 0; i < KV; i++) {
-                const float4 g = reinterpret_cast<const float4*>(p.gamma)[i * 64 + lane];
-                const float4 be = reinterpret_cast<const float4*>(p.beta)[i * 64 + lane];
-                h[i] = make_float4(g.x * h[i].x * inv_std + be.x, g.y * h[i].y * inv_std + be.y,
-                                   g.z * h[i].z * inv_std + be.z, g.w * h[i].w * inv_std + be.w);
-            }
-        }
+        norm_in_registers<KV, PRO>(h, p.gamma, p.beta, K, lane);
 #pragma unroll
         for (int r = 0; r < R; r++) {
             float a = 0.0f;

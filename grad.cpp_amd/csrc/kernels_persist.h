@@ -1,0 +1,712 @@
+// Persistent batch-1 decoder: ONE kernel launch runs a whole run of steps
+// (prompt tokens, then pick + step rounds), because at 69M parameters a step is
+// ~40 dependent projections of a few microseconds each and a kernel launch per
+// projection costs more than the projection.
+//
+// One workgroup per compute unit stays resident.  Inside a step the phases
+//   norm+QKV -> attention -> W_o+residual -> norm+FFN1 -> FFN2+residual  (per layer)
+//   -> final norm + logits -> pick
+// hand their outputs to the next phase through "cells": 8-byte {value, tag}
+// pairs written and read with single device-scope accesses, so a value and the
+// tag that says which (step, layer, phase) produced it always travel together.
+// A consumer polls the cells it needs until every tag matches; there is no
+// separate barrier.  Polling is bounded and watches an abort flag, so every
+// wavefront leaves the kernel even if a producer never shows up.
+//
+// The arithmetic per phase is the same as the one-kernel-per-op path
+// (kernels_gemv.h, kernels_attn.h), i.e. src/transformer/inference.cpp:150-258.
+#pragma once
+
+#include "kernels_common.h"
+#include "kernels_gemv.h"
+#include "kernels_pick.h"
+
+namespace gh {
+
+constexpr int kPersistThreads = 512;
+constexpr int kPersistWaves = kPersistThreads / 64;
+
+struct Cell {
+    float v;
+    unsigned tag;
+};
+
+struct LayerPtrs {
+    const float *wqkv, *bqkv, *wo, *bo, *w1, *b1, *w2, *b2, *g1, *be1, *g2, *be2;
+};
+
+struct PersistCtl {
+    unsigned abort;     // set by any workgroup that gave up waiting
+    unsigned where;     // phase tag it was waiting for (diagnostics)
+    unsigned pad[30];
+    unsigned arrive[16 * 32];  // logits-complete counters, one per 128-byte line
+};
+
+struct PersistParams {
+    const float* E;
+    const float* P;
+    const LayerPtrs* layers;  // device array
+    const float *gf, *bf, *rope_cos, *rope_sin;
+    int d, F, V, L, H;
+    KvLayout kv;
+    Cell *xa, *xb, *q, *kn, *vn, *at, *hid, *tokc;
+    float* logits;     // [V]
+    float* logit_log;  // [steps][V] or nullptr
+    PersistCtl* ctl;
+    int* hist;  // token history of the sequence
+    int pos0;          // cache positions already filled
+    int n_prompt;      // steps whose token is hist[pos0 + s]
+    int n_steps;       // step() calls in this launch
+    int n_picks;       // picks in this launch
+    int start_with_pick;  // the first pick uses the logits already in memory
+    unsigned epoch;    // tag base of this launch; (epoch + s) never repeats in a session
+    unsigned arrive_base;  // logits phases completed before this launch
+    PickParams pick;
+    unsigned spin_limit;
+    unsigned long long* prof;  // optional: phase-end timestamps of workgroup 0 (100 MHz clock)
+    int prof_cap;
+};
+
+__device__ __forceinline__ void cell_put(Cell* c, float v, unsigned tag) {
+    const unsigned long long w =
+        (static_cast<unsigned long long>(tag) << 32) | static_cast<unsigned long long>(__float_as_uint(v));
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(c), w, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ bool cell_get(const Cell* c, unsigned tag, float& v) {
+    const unsigned long long w = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(c),
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v = __uint_as_float(static_cast<unsigned>(w));
+    return static_cast<unsigned>(w >> 32) == tag;
+}
+
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Workgroup-wide: waits until cells [0, n) carry `tag`, copying the values to
+// dst (LDS).  Returns false when the wait was abandoned (the kernel must exit).
+__device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float* dst,
+                                    const PersistParams& p) {
+    const __amdgpu_buffer_rsrc_t rs = make_buffer(src, static_cast<unsigned>(n) * 8u);
+    const int itag = static_cast<int>(tag);
+    unsigned spins = 0;
+    for (;;) {
+        bool ok = true;
+        // two cells per 16-byte load, all of a thread's loads in flight together
+        for (int i = 2 * threadIdx.x; i < n; i += 2 * blockDim.x) {
+            const v4i w = coherent_load16(rs, static_cast<unsigned>(i) * 8u);
+            ok = ok && w.y == itag && (i + 1 >= n || w.w == itag);
+            dst[i] = __int_as_float(w.x);
+            if (i + 1 < n) dst[i + 1] = __int_as_float(w.z);
+        }
+        if (__syncthreads_and(ok)) return true;
+        ++spins;
+        bool give_up = spins > p.spin_limit;
+        if ((spins & 63u) == 0u)
+            give_up = give_up || __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+        if (__syncthreads_or(give_up)) {
+            if (threadIdx.x == 0) {
+                __hip_atomic_store(&p.ctl->where, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            return false;
+        }
+    }
+}
+
+// One pick by workgroup 0 (text_gen.cpp:48-61 / :80-86): waits until every
+// workgroup's logits rows have landed, picks, records the token in the history
+// and publishes it in the token cell.  The other workgroups return at once and
+// learn the token from the cell.  False: the wait was abandoned.
+__device__ inline bool persist_pick(const PersistParams& p, float* lds, int i_pick,
+                                    unsigned arrive_gen, unsigned tok_tag, bool wait_logits) {
+    if (blockIdx.x != 0) return true;
+    __shared__ unsigned total;
+    const int tid = threadIdx.x;
+    if (p.prof && i_pick < 1024 && tid == 0) p.prof[p.prof_cap / 2 + 4 * i_pick + 2] = __builtin_amdgcn_s_memrealtime();
+    if (wait_logits) {
+        unsigned spins = 0;
+        for (;;) {
+            unsigned v = 0;
+            if (tid < 16)
+                v = __hip_atomic_load(&p.ctl->arrive[tid * 32], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid < 64) {
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+            }
+            if (tid == 0) total = v;
+            __syncthreads();
+            const bool done = total >= arrive_gen * gridDim.x;
+            __syncthreads();
+            if (done) break;
+            const bool aborted = (spins & 63u) == 63u
+                                 && __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+            if (__syncthreads_or(++spins > p.spin_limit || aborted)) {
+                if (tid == 0) {
+                    __hip_atomic_store(&p.ctl->where, 0xFFFFFFFEu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                return false;
+            }
+        }
+    }
+    unsigned long long* pp = (p.prof && i_pick < 1024) ? p.prof + p.prof_cap / 2 + 4 * i_pick : nullptr;
+    if (pp && tid == 0) pp[0] = __builtin_amdgcn_s_memrealtime();
+    PickParams pk = p.pick;
+    pk.n_hist = p.pick.n_hist + i_pick;
+    pk.pick_idx = p.pick.pick_idx + i_pick;
+    pk.dbg = (p.prof && i_pick == 100) ? p.prof + p.prof_cap - 16 : nullptr;
+#ifndef PROBE_NO_PICK
+    const int chosen = pick_lds_body(pk, 0, lds, true);
+#else
+    const int chosen = 0;
+#endif
+    if (tid == 0) {
+        __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        cell_put(p.tokc, __int_as_float(chosen), tok_tag);
+        if (pp) pp[1] = __builtin_amdgcn_s_memrealtime();
+    }
+    return true;
+}
+
+template <int KV>
+__device__ __forceinline__ void load_row(const float* W, int row, int K, int lane, float4 (&w)[KV]) {
+    const float4* wr = reinterpret_cast<const float4*>(W + static_cast<size_t>(row) * K);
+#pragma unroll
+    for (int i = 0; i < KV; i++) w[i] = wr[i * 64 + lane];
+}
+
+template <int KV>
+__device__ __forceinline__ float dot_row(const float4 (&w)[KV], const float4 (&h)[KV]) {
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < KV; i++) a += dot4(w[i], h[i]);
+    return wave_sum(a);
+}
+
+// Register-resident norm parameters of one lane: the gamma (and beta) float4s
+// that line up with its slice of the row.
+template <int KV>
+struct NormRegs {
+    float4 g[KV];
+    float4 b[KV];
+};
+
+template <int KV, int PRO>
+__device__ __forceinline__ void load_norm(const float* gamma, const float* beta, int lane, NormRegs<KV>& n) {
+    if constexpr (PRO != PRO_PLAIN) {
+#pragma unroll
+        for (int i = 0; i < KV; i++) n.g[i] = reinterpret_cast<const float4*>(gamma)[i * 64 + lane];
+    }
+    if constexpr (PRO == PRO_LAYERNORM) {
+#pragma unroll
+        for (int i = 0; i < KV; i++) n.b[i] = reinterpret_cast<const float4*>(beta)[i * 64 + lane];
+    }
+}
+
+// This lane's slice of the input vector held in LDS, normalised with preloaded
+// gamma / beta (layer_norm_row, inference.cpp:30-58).
+template <int KV, int PRO>
+__device__ __forceinline__ void load_input(const float* xs, const NormRegs<KV>& n, int lane, float4 (&h)[KV]) {
+    constexpr int K = KV * 256;
+#pragma unroll
+    for (int i = 0; i < KV; i++) h[i] = reinterpret_cast<const float4*>(xs)[i * 64 + lane];
+    if constexpr (PRO == PRO_RMSNORM) {
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < KV; i++) ss += dot4(h[i], h[i]);
+        const float r = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(K) + kNormEps);
+#pragma unroll
+        for (int i = 0; i < KV; i++)
+            h[i] = make_float4(n.g[i].x * h[i].x * r, n.g[i].y * h[i].y * r, n.g[i].z * h[i].z * r,
+                               n.g[i].w * h[i].w * r);
+    } else if constexpr (PRO == PRO_LAYERNORM) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < KV; i++) sum += (h[i].x + h[i].y) + (h[i].z + h[i].w);
+        const float mean = wave_sum(sum) / static_cast<float>(K);
+        float var = 0.0f;
+#pragma unroll
+        for (int i = 0; i < KV; i++) {
+            h[i] = make_float4(h[i].x - mean, h[i].y - mean, h[i].z - mean, h[i].w - mean);
+            var += dot4(h[i], h[i]);
+        }
+        const float inv_std = 1.0f / sqrtf(wave_sum(var) / static_cast<float>(K) + kNormEps);
+#pragma unroll
+        for (int i = 0; i < KV; i++)
+            h[i] = make_float4(n.g[i].x * h[i].x * inv_std + n.b[i].x, n.g[i].y * h[i].y * inv_std + n.b[i].y,
+                               n.g[i].z * h[i].z * inv_std + n.b[i].z, n.g[i].w * h[i].w * inv_std + n.b[i].w);
+    }
+}
+
+// Everything phase A (norm1 + QKV) needs that does not depend on the
+// activations: two weight rows, the norm parameters, the biases and the
+// rotation of this position.  Loaded one exchange ahead of its use.
+template <int KD, int PRO>
+struct QkvOperands {
+    float4 w0[KD], w1[KD];
+    NormRegs<KD> n;
+    float b0, b1, cs, sn;
+};
+
+template <int KD, int PRO, bool MODERN>
+__device__ __forceinline__ void load_qkv_operands(const PersistParams& p, const LayerPtrs& w, int item,
+                                                  int pos, int lane, QkvOperands<KD, PRO>& o) {
+    constexpr int D = KD * 256, HS = 64;
+    const int row = 2 * item;
+    load_row<KD>(w.wqkv, row, D, lane, o.w0);
+    load_row<KD>(w.wqkv, row + 1, D, lane, o.w1);
+    load_norm<KD, PRO>(w.g1, w.be1, lane, o.n);
+    o.b0 = w.bqkv[row];
+    o.b1 = w.bqkv[row + 1];
+    o.cs = 1.0f;
+    o.sn = 0.0f;
+    if (MODERN && row < 2 * D) {
+        const int j = ((row % D) % HS) >> 1;
+        o.cs = p.rope_cos[pos * (HS / 2) + j];
+        o.sn = p.rope_sin[pos * (HS / 2) + j];
+    }
+}
+
+// KD = d_model / 256, KF = FFN width / 256; head size 64; context <= 512.
+template <int KD, int KF, bool MODERN>
+__global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const PersistParams p) {
+    extern __shared__ float lds[];
+    constexpr int D = KD * 256, F = KF * 256, HS = 64;
+    constexpr int PRO = MODERN ? PRO_RMSNORM : PRO_LAYERNORM;
+    constexpr int RL = 8;  // logits rows per wavefront item
+    float* xs = lds;                      // [D] residual stream of this step
+    float* vin = lds + D;                 // [max(D, F)] attention output / FFN hidden
+    float* ascr = vin + (F > D ? F : D);  // attention scratch: q, k, v of the head + wave partials
+    int* ptab = reinterpret_cast<int*>(ascr + 192 + kPersistWaves * 68);  // [pages_per_seq]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wg = blockIdx.x, G = gridDim.x;
+    const int V = p.V, L = p.L, H = p.H;
+    const int stride = G * kPersistWaves;  // wavefronts in the grid
+    const int first = wg + G * wave;       // item i of a phase goes to workgroup i % G
+    int i_pick = 0;
+    unsigned arrive_gen = p.arrive_base;
+    int n_stamp = 0;
+    auto stamp = [&]() {
+        if (p.prof && wg == 0 && tid == 0 && n_stamp < p.prof_cap) p.prof[n_stamp] = __builtin_amdgcn_s_memrealtime();
+        n_stamp++;
+    };
+    stamp();
+
+    // The sequence's page table never changes while the kernel runs.
+    for (int i = tid; i < p.kv.pages_per_seq; i += kPersistThreads) ptab[i] = p.kv.page_table[i];
+    __syncthreads();
+    auto kv_at = [&](int layer, int which, int head, int t) -> size_t {
+        const int page = ptab[t >> p.kv.page_shift];
+        const int slot = t & ((1 << p.kv.page_shift) - 1);
+        const size_t run = ((static_cast<size_t>(layer) * p.kv.n_pages + page) * 2 + which) * H + head;
+        return ((run << p.kv.page_shift) + slot) * HS;
+    };
+
+    if (p.start_with_pick && p.n_picks > 0) {
+        const unsigned tt = (p.epoch * static_cast<unsigned>(L + 1) + static_cast<unsigned>(L)) * 8u + 6u;
+        if (!persist_pick(p, lds, i_pick, arrive_gen, tt, false)) return;
+        i_pick++;
+        if (wg == 0) {
+            // the pick used the whole LDS; restore the page table
+            __syncthreads();
+            for (int i = tid; i < p.kv.pages_per_seq; i += kPersistThreads) ptab[i] = p.kv.page_table[i];
+            __syncthreads();
+        }
+    }
+
+    constexpr int NQKV = 3 * D / 2;  // phase A items: pairs of rows
+    const bool has_qkv = first < NQKV;
+
+    for (int s = 0; s < p.n_steps; s++) {
+        const int pos = p.pos0 + s;
+        const unsigned sb = (p.epoch + 1u + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1);
+        auto tag_of = [&](int layer, int ph) {
+            return (sb + static_cast<unsigned>(layer)) * 8u + static_cast<unsigned>(ph) + 1u;
+        };
+        const bool want_logits = (s >= p.n_prompt - 1) || p.logit_log != nullptr || s == p.n_steps - 1;
+
+        // Operands of layer 0's QKV are fetched while the token arrives.
+        QkvOperands<KD, PRO> qo;
+        {
+            const LayerPtrs w0l = p.layers[0];
+            if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, w0l, first, pos, lane, qo);
+        }
+
+        // ---- token and embedding (inference.cpp:159-182)
+        int tok;
+        if (s < p.n_prompt) {
+            tok = p.hist[pos];
+        } else {
+            // the pick that followed step s-1 (or opened the launch)
+            const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
+                                 + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
+            if (!gather_cells(p.tokc, 1, tt, ascr, p)) return;
+            tok = __float_as_int(ascr[0]);
+            __syncthreads();
+        }
+        for (int j = tid; j < D; j += kPersistThreads) {
+            float v = p.E[static_cast<size_t>(tok) * D + j];
+            if (!MODERN) v += p.P[static_cast<size_t>(pos) * D + j];
+            xs[j] = v;
+        }
+        __syncthreads();
+
+        for (int l = 0; l < L; l++) {
+            const LayerPtrs w = p.layers[l];
+
+            // ===== phase A: norm1 + QKV (+bias, RoPE) -> q / new k / new v cells and the cache
+            for (int item = first; item < NQKV; ) {
+                const int row = 2 * item;
+                float4 h[KD];
+                load_input<KD, PRO>(xs, qo.n, lane, h);
+                float a = dot_row<KD>(qo.w0, h) + qo.b0;
+                float c = dot_row<KD>(qo.w1, h) + qo.b1;
+                if (lane == 0) {
+                    const int sec = row / D, col = row - sec * D;
+                    if (MODERN && sec < 2) {
+                        const float ra = a * qo.cs - c * qo.sn;
+                        const float rc = a * qo.sn + c * qo.cs;
+                        a = ra;
+                        c = rc;
+                    }
+                    const unsigned t = tag_of(l, 0);
+                    if (sec == 0) {
+                        cell_put(p.q + col, a, t);
+                        cell_put(p.q + col + 1, c, t);
+                    } else {
+                        Cell* dst = (sec == 1 ? p.kn : p.vn) + col;
+                        cell_put(dst, a, t);
+                        cell_put(dst + 1, c, t);
+                        const int head = col / HS, jj = col - head * HS;
+                        float* cr = p.kv.pool + kv_at(l, sec - 1, head, pos) + jj;
+                        coherent_store(cr, a);
+                        coherent_store(cr + 1, c);
+                    }
+                }
+                item += stride;
+                if (item < NQKV) load_qkv_operands<KD, PRO, MODERN>(p, w, item, pos, lane, qo);
+            }
+            stamp();
+
+            // ===== phase B: attention of one head per workgroup (inference.cpp:211-225)
+#ifndef PROBE_NO_ATTN
+            if (wg < H) {
+                const int hd = wg;
+                float* qkv = ascr;         // [3][64]: q, key and value of the current position
+                float* part = ascr + 192;  // [waves][68]: m, l, pad, pad, acc[64]
+                const int ctx = pos + 1;
+                // positions are dealt to the wavefronts in runs of `chunk` (a multiple of 4, <= 64)
+                const int chunk = min(64, (((ctx + kPersistWaves - 1) / kPersistWaves) + 3) & ~3);
+                const int sub = lane >> 4, dl = lane & 15;
+                const int t0 = wave * chunk;
+                // Cached rows do not depend on this step's q: the first 32 positions of
+                // the run are fetched before waiting for q (all of it for contexts <= 256).
+                const float* pool = p.kv.pool;
+                float4 k4[8], v4[8];
+#pragma unroll
+                for (int it = 0; it < 8; it++) {
+                    const int tt = t0 + it * 4 + sub;
+                    k4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    v4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (it * 4 < chunk && tt < pos) {
+                        const unsigned ko = static_cast<unsigned>(kv_at(l, 0, hd, tt)) + dl * 4;
+                        const unsigned vo = static_cast<unsigned>(kv_at(l, 1, hd, tt)) + dl * 4;
+                        k4[it] = *reinterpret_cast<const float4*>(pool + ko);
+                        v4[it] = *reinterpret_cast<const float4*>(pool + vo);
+                    }
+                }
+                // q, new key, new value of this head: one wait for all three
+                {
+                    const unsigned t = tag_of(l, 0);
+                    unsigned spins = 0;
+                    for (;;) {
+                        bool ok = true;
+                        if (tid < 96) {
+                            const int seg = tid >> 5, j = (tid & 31) * 2;
+                            const Cell* src = (seg == 0 ? p.q : seg == 1 ? p.kn : p.vn) + hd * HS;
+                            const v4i w = coherent_load16(make_buffer(src, HS * 8u), static_cast<unsigned>(j) * 8u);
+                            ok = w.y == static_cast<int>(t) && w.w == static_cast<int>(t);
+                            qkv[seg * 64 + j] = __int_as_float(w.x);
+                            qkv[seg * 64 + j + 1] = __int_as_float(w.z);
+                        }
+                        if (__syncthreads_and(ok)) break;
+                        ++spins;
+                        bool give_up = spins > p.spin_limit;
+                        if ((spins & 63u) == 0u)
+                            give_up = give_up || __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+                        if (__syncthreads_or(give_up)) {
+                            if (tid == 0) {
+                                __hip_atomic_store(&p.ctl->where, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            }
+                            return;
+                        }
+                    }
+                }
+                const float4 q4 = reinterpret_cast<const float4*>(qkv)[dl];
+                float m = -INFINITY, lsum = 0.0f;
+                float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+                // Two batches of 8 iterations (32 positions); softmax state is merged online.
+                for (int batch = 0; batch < 2; batch++) {
+                    if (batch * 32 >= chunk) break;
+                    if (batch == 1) {
+#pragma unroll
+                        for (int it = 0; it < 8; it++) {
+                            const int tt = t0 + 32 + it * 4 + sub;
+                            k4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+                            v4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+                            if (32 + it * 4 < chunk && tt < pos) {
+                                const unsigned ko = static_cast<unsigned>(kv_at(l, 0, hd, tt)) + dl * 4;
+                                const unsigned vo = static_cast<unsigned>(kv_at(l, 1, hd, tt)) + dl * 4;
+                                k4[it] = *reinterpret_cast<const float4*>(pool + ko);
+                                v4[it] = *reinterpret_cast<const float4*>(pool + vo);
+                            }
+                        }
+                    }
+                    float sc[8];
+#pragma unroll
+                    for (int it = 0; it < 8; it++) {
+                        const int rel = batch * 32 + it * 4 + sub;
+                        const int tt = t0 + rel;
+                        const bool in_run = rel < chunk;
+                        if (in_run && tt == pos) {
+                            k4[it] = reinterpret_cast<const float4*>(qkv + 64)[dl];
+                            v4[it] = reinterpret_cast<const float4*>(qkv + 128)[dl];
+                        }
+                        float sdot = dot4(q4, k4[it]);
+                        sdot += __shfl_xor(sdot, 1, kWave);
+                        sdot += __shfl_xor(sdot, 2, kWave);
+                        sdot += __shfl_xor(sdot, 4, kWave);
+                        sdot += __shfl_xor(sdot, 8, kWave);
+                        sc[it] = (in_run && tt < ctx) ? sdot * 0.125f : -INFINITY;  // 1/sqrt(64)
+                    }
+                    float mb = sc[0];
+#pragma unroll
+                    for (int it = 1; it < 8; it++) mb = fmaxf(mb, sc[it]);
+                    mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
+                    mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
+                    const float mn = fmaxf(m, mb);
+                    if (mn > -INFINITY) {
+                        const float f = expf(m - mn);  // 0 on the first batch (m = -inf)
+                        lsum *= f;
+                        acc.x *= f;
+                        acc.y *= f;
+                        acc.z *= f;
+                        acc.w *= f;
+#pragma unroll
+                        for (int it = 0; it < 8; it++) {
+                            const float e = expf(sc[it] - mn);  // exp(-inf) = 0 for unused slots
+                            lsum += e;
+                            acc.x += e * v4[it].x;
+                            acc.y += e * v4[it].y;
+                            acc.z += e * v4[it].z;
+                            acc.w += e * v4[it].w;
+                        }
+                        m = mn;
+                    }
+                }
+                // lsum and acc hold this lane group's share; sum the four groups
+                lsum += __shfl_xor(lsum, 16, kWave);
+                lsum += __shfl_xor(lsum, 32, kWave);
+#pragma unroll
+                for (int o = 16; o < 64; o <<= 1) {
+                    acc.x += __shfl_xor(acc.x, o, kWave);
+                    acc.y += __shfl_xor(acc.y, o, kWave);
+                    acc.z += __shfl_xor(acc.z, o, kWave);
+                    acc.w += __shfl_xor(acc.w, o, kWave);
+                }
+                if (lane < 16) reinterpret_cast<float4*>(part + wave * 68 + 4)[lane] = acc;
+                if (lane == 0) {
+                    part[wave * 68] = m;
+                    part[wave * 68 + 1] = lsum;
+                }
+                __syncthreads();
+                if (tid < HS) {
+                    float M = -INFINITY;
+                    for (int w8 = 0; w8 < kPersistWaves; w8++) M = fmaxf(M, part[w8 * 68]);
+                    float Lsum = 0.0f, o = 0.0f;
+                    for (int w8 = 0; w8 < kPersistWaves; w8++) {
+                        const float f = expf(part[w8 * 68] - M);  // 0 for wavefronts without positions
+                        Lsum += part[w8 * 68 + 1] * f;
+                        o += part[w8 * 68 + 4 + tid] * f;
+                    }
+                    cell_put(p.at + hd * HS + tid, o * (1.0f / Lsum), tag_of(l, 1));
+                }
+                __syncthreads();
+            }
+#endif
+            stamp();
+
+            // ===== phase C: x += b_o + attn @ W_o
+            {
+                float4 w0[KD];
+                float bo = 0.0f;
+                if (first < D) {
+                    load_row<KD>(w.wo, first, D, lane, w0);
+                    bo = w.bo[first];
+                }
+                if (!gather_cells(p.at, D, tag_of(l, 1), vin, p)) return;
+                for (int row = first; row < D; ) {
+                    float4 h[KD];
+#pragma unroll
+                    for (int i = 0; i < KD; i++) h[i] = reinterpret_cast<const float4*>(vin)[i * 64 + lane];
+                    const float a = dot_row<KD>(w0, h);
+                    if (lane == 0) cell_put(p.xb + row, (xs[row] + bo) + a, tag_of(l, 2));
+                    row += stride;
+                    if (row < D) {
+                        load_row<KD>(w.wo, row, D, lane, w0);
+                        bo = w.bo[row];
+                    }
+                }
+            }
+            stamp();
+
+            // ===== phase D: norm2 + FFN1 (SwiGLU or GELU) -> hidden cells
+            {
+                constexpr int NIT = MODERN ? F : F / 2;  // pairs of weight rows
+                float4 w0[KD], w1[KD];
+                NormRegs<KD> n2;
+                float b0 = 0.0f, b1 = 0.0f;
+                if (first < NIT) {
+                    load_row<KD>(w.w1, 2 * first, D, lane, w0);
+                    load_row<KD>(w.w1, 2 * first + 1, D, lane, w1);
+                    load_norm<KD, PRO>(w.g2, w.be2, lane, n2);
+                    if (!MODERN) {
+                        b0 = w.b1[2 * first];
+                        b1 = w.b1[2 * first + 1];
+                    }
+                }
+                __syncthreads();  // every wave is done reading xs (phase C)
+                if (!gather_cells(p.xb, D, tag_of(l, 2), xs, p)) return;
+                for (int item = first; item < NIT; ) {
+                    float4 h[KD];
+                    load_input<KD, PRO>(xs, n2, lane, h);
+                    const float a = dot_row<KD>(w0, h);
+                    const float c = dot_row<KD>(w1, h);
+                    if (lane == 0) {
+                        const unsigned t = tag_of(l, 3);
+                        if (MODERN) {
+                            cell_put(p.hid + item, c * silu(a), t);
+                        } else {
+                            cell_put(p.hid + 2 * item, gelu_tanh(a + b0), t);
+                            cell_put(p.hid + 2 * item + 1, gelu_tanh(c + b1), t);
+                        }
+                    }
+                    item += stride;
+                    if (item < NIT) {
+                        load_row<KD>(w.w1, 2 * item, D, lane, w0);
+                        load_row<KD>(w.w1, 2 * item + 1, D, lane, w1);
+                        if (!MODERN) {
+                            b0 = w.b1[2 * item];
+                            b1 = w.b1[2 * item + 1];
+                        }
+                    }
+                }
+            }
+            stamp();
+
+            // ===== phase E: x += (b2 +) hidden @ W2 -> next layer's input cells
+            {
+                float4 w0[KF];
+                float b2 = 0.0f;
+                if (first < D) {
+                    load_row<KF>(w.w2, first, F, lane, w0);
+                    if (!MODERN) b2 = w.b2[first];
+                }
+                if (!gather_cells(p.hid, F, tag_of(l, 3), vin, p)) return;
+                for (int row = first; row < D; ) {
+                    float4 h[KF];
+#pragma unroll
+                    for (int i = 0; i < KF; i++) h[i] = reinterpret_cast<const float4*>(vin)[i * 64 + lane];
+                    const float a = dot_row<KF>(w0, h);
+                    if (lane == 0) cell_put(p.xa + row, (xs[row] + b2) + a, tag_of(l, 4));
+                    row += stride;
+                    if (row < D) {
+                        load_row<KF>(w.w2, row, F, lane, w0);
+                        if (!MODERN) b2 = w.b2[row];
+                    }
+                }
+            }
+            stamp();
+
+            // ===== the next consumer of x is layer l+1's QKV: its operands are
+            // fetched while x is still being exchanged.
+            if (l + 1 < L) {
+                const LayerPtrs wn = p.layers[l + 1];
+                if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, wn, first, pos, lane, qo);
+                __syncthreads();  // xs is overwritten next
+                if (!gather_cells(p.xa, D, tag_of(l, 4), xs, p)) return;
+            }
+        }
+
+#ifndef PROBE_NO_LOGITS
+        if (want_logits) {
+            // ===== final norm + logits = h @ E^T (inference.cpp:251-254); the rows of
+            // E are fetched while the last layer's x is still being exchanged.
+            const int nitems = (V + RL - 1) / RL;
+            float4 wr[RL][KD];
+            NormRegs<KD> nf;
+            load_norm<KD, PRO>(p.gf, p.bf, lane, nf);
+            if (first < nitems) {
+#pragma unroll
+                for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(first * RL + r, V - 1), D, lane, wr[r]);
+            }
+            __syncthreads();
+            if (!gather_cells(p.xa, D, tag_of(L - 1, 4), xs, p)) return;
+            stamp();
+            float4 h[KD];
+            load_input<KD, PRO>(xs, nf, lane, h);
+            for (int item = first; item < nitems; ) {
+                float out[RL];
+#pragma unroll
+                for (int r = 0; r < RL; r++) out[r] = dot_row<KD>(wr[r], h);
+                if (lane == 0) {
+#pragma unroll
+                    for (int r = 0; r < RL; r++) {
+                        const int row = item * RL + r;
+                        if (row < V) {
+                            coherent_store(p.logits + row, out[r]);
+                            if (p.logit_log) p.logit_log[static_cast<size_t>(s) * V + row] = out[r];
+                        }
+                    }
+                }
+                item += stride;
+                if (item < nitems) {
+#pragma unroll
+                    for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(item * RL + r, V - 1), D, lane, wr[r]);
+                }
+            }
+            // this workgroup's rows are out: signal
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            arrive_gen++;
+            if (tid == 0)
+                __hip_atomic_fetch_add(&p.ctl->arrive[(wg & 15) * 32], 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        } else
+#endif
+        {
+            // nobody needs this step's logits: the last x stays in its cells
+            stamp();
+        }
+        stamp();
+
+        // ===== pick (decode rounds only)
+        if (i_pick < p.n_picks && s >= p.n_prompt - 1) {
+            const unsigned tt = (sb + static_cast<unsigned>(L)) * 8u + 7u;
+            if (!persist_pick(p, lds, i_pick, arrive_gen, tt, true)) return;
+            i_pick++;
+            if (wg == 0) {
+                __syncthreads();
+                for (int i = tid; i < p.kv.pages_per_seq; i += kPersistThreads) ptab[i] = p.kv.page_table[i];
+                __syncthreads();
+            }
+        }
+        stamp();
+    }
+}
+
+}  // namespace gh

@@ -36,6 +36,7 @@ struct PickParams {
     unsigned seed_lo, seed_hi;
     int sort_cap;  // floats of LDS available for the descending sort (power of two)
     int* err;      // set to 1 when top-p needs a sort larger than sort_cap
+    unsigned long long* dbg;  // optional timestamps (developer aid)
 };
 
 __device__ __forceinline__ unsigned mulhi32(unsigned a, unsigned b) { return __umulhi(a, b); }
@@ -418,9 +419,29 @@ __device__ inline float kth_largest_lds(const float* v, int n, int k, unsigned* 
     for (int shift = 24; shift >= 0; shift -= 8) {
         for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0u;
         __syncthreads();
-        for (int i = threadIdx.x; i < n; i += blockDim.x) {
-            const unsigned key = float_key(v[i]);
-            if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        // Keys cluster in a few bins (same sign and exponent), so lanes that hit
+        // the same bin are counted with one atomic per wavefront.
+        const int n_round = (n + blockDim.x - 1) / blockDim.x * blockDim.x;
+        for (int i = threadIdx.x; i < n_round; i += blockDim.x) {
+            unsigned key = 0u;
+            bool active = false;
+            if (i < n) {
+                key = float_key(v[i]);
+                active = (key & mask) == prefix;
+            }
+            const unsigned bin = (key >> shift) & 255u;
+            // up to two crowded bins are counted once per wavefront; what is left is
+            // spread out and goes through per-lane atomics
+            unsigned long long todo = __ballot(active);
+            for (int rep = 0; rep < 2 && todo; rep++) {
+                const int leader = __ffsll(static_cast<long long>(todo)) - 1;
+                const unsigned lb = __builtin_amdgcn_readlane(bin, leader);
+                const unsigned long long same = __ballot(active && bin == lb);
+                if ((threadIdx.x & 63) == leader) atomicAdd(&hist[lb], static_cast<unsigned>(__popcll(same)));
+                if (bin == lb) active = false;
+                todo &= ~same;
+            }
+            if (active) atomicAdd(&hist[bin], 1u);
         }
         __syncthreads();
         if (threadIdx.x < 64) select_bin_wave(hist, remaining, bcast);
@@ -430,6 +451,64 @@ __device__ inline float kth_largest_lds(const float* v, int n, int k, unsigned* 
         remaining = static_cast<int>(bcast[1]);
     }
     return key_float(prefix);
+}
+
+// The k-th largest of v[0..n) for small k, without passes over radix digits:
+// the k-th largest of the per-thread maxima is a lower bound T of the answer (at
+// least k elements are >= T), the elements >= T are few, and the answer is the
+// k-th largest of those.  Falls back to the radix select when k exceeds the
+// workgroup size or `work` (work_cap floats) cannot hold 2 * blockDim.x + 16.
+__device__ inline float kth_largest_block(const float* v, int n, int k, float* work, int work_cap,
+                                          unsigned* hist, unsigned* bcast, int* ishare) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+    if (k > nt || work_cap < 2 * nt + 16) return kth_largest_lds(v, n, k, hist, bcast);
+    float mx = -INFINITY;
+    for (int i = tid; i < n; i += nt) mx = fmaxf(mx, v[i]);
+    work[tid] = mx;
+    if (tid == 0) ishare[1] = 0;
+    __syncthreads();
+    {
+        // nt is a multiple of 64: reads in groups of 16 keep the LDS pipeline full
+        int rank = 0;
+        for (int j0 = 0; j0 < nt; j0 += 16) {
+            float o[16];
+#pragma unroll
+            for (int q = 0; q < 16; q++) o[q] = work[j0 + q];
+#pragma unroll
+            for (int q = 0; q < 16; q++) rank += (o[q] > mx) || (o[q] == mx && j0 + q < tid);
+        }
+        if (rank == k - 1) bcast[0] = __float_as_uint(mx);
+    }
+    __syncthreads();
+    const float T = __uint_as_float(bcast[0]);
+    float* cand = work + nt;  // [nt + 16]
+    for (int i = tid; i < n; i += nt) {
+        const float x = v[i];
+        if (x >= T) {
+            const int slot = atomicAdd(&ishare[1], 1);
+            if (slot < nt) cand[slot] = x;
+        }
+    }
+    __syncthreads();
+    const int c = ishare[1];
+    __syncthreads();
+    if (c > nt) return kth_largest_lds(v, n, k, hist, bcast);
+    {
+        const float mine = tid < c ? cand[tid] : -INFINITY;
+        for (int j = c + tid; j < ((c + 15) & ~15); j += nt) cand[j] = -INFINITY;  // pad to 16
+        __syncthreads();
+        int rank = 0;
+        for (int j0 = 0; j0 < c; j0 += 16) {
+            float o[16];
+#pragma unroll
+            for (int q = 0; q < 16; q++) o[q] = cand[j0 + q];
+#pragma unroll
+            for (int q = 0; q < 16; q++) rank += (o[q] > mine) || (o[q] == mine && j0 + q < tid);
+        }
+        if (tid < c && rank == k - 1) bcast[0] = __float_as_uint(mine);
+    }
+    __syncthreads();
+    return __uint_as_float(bcast[0]);
 }
 
 // Ascending bitonic sort of ints, n2 a power of two.
@@ -464,10 +543,101 @@ __device__ __forceinline__ int block_sum_int(int v, int* scratch) {
     return r;
 }
 
+// The sampler's tail for at most 64 survivors of the top-k cut, run by one
+// wavefront with lane i holding survivor i in index order: softmax, top-p,
+// renormalisation and the inverse-CDF walk (text_gen.cpp:156-208).  Every sum the
+// reference forms in index or sorted order is formed in that same order here
+// (entries cut by top-k are exact zeros there and add nothing).
+__device__ inline int pick_small_wave(const float* val, const int* cidx, int S, float top_p, float u,
+                                      int V, float* scratch /* >= 256 floats */) {
+    const int lane = threadIdx.x & 63;
+    int* sidx = reinterpret_cast<int*>(scratch);  // [64] survivor indices, ascending
+    float* se = scratch + 64;                     // [64] values in index order, zero padded
+    float* sp = scratch + 128;                    // [64] probabilities, descending, zero padded
+    // index order (all loops run a fixed 64 rounds over padded arrays so that
+    // their LDS reads can be issued together)
+    const int my = lane < S ? cidx[lane] : 0x7FFFFFFF;
+    sidx[lane] = my;
+    __builtin_amdgcn_wave_barrier();
+    int rank = 0;
+#pragma unroll
+    for (int j = 0; j < 64; j++) rank += (sidx[j] < my);
+    __builtin_amdgcn_wave_barrier();
+    if (lane < S) sidx[rank] = my;
+    __builtin_amdgcn_wave_barrier();
+    const int idx = lane < S ? sidx[lane] : 0;
+    const float v = lane < S ? val[idx] : -INFINITY;
+    const float m = wave_max(v);
+    const float e = lane < S ? expf(v - m) : 0.0f;
+    se[lane] = e;
+    __builtin_amdgcn_wave_barrier();
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 64; j++) sum += se[j];  // index order; padding adds exact zeros
+    float pr = e * (1.0f / sum);
+    bool keep = lane < S && pr > 0.0f;
+    __builtin_amdgcn_wave_barrier();
+    se[lane] = pr;
+    __builtin_amdgcn_wave_barrier();
+    if (top_p < 1.0f) {
+        int r = 0;
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+            const float pj = se[j];
+            r += (pj > pr) || (pj == pr && j < lane);
+        }
+        sp[r] = pr;  // ranks are a permutation of 0..63: padding zeros land at the end
+        __builtin_amdgcn_wave_barrier();
+        float cumulative = 0.0f, cutoff = 0.0f;
+        bool found = false;
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+            const float x = sp[j];
+            cumulative += x;
+            if (!found && j < S && cumulative >= top_p) {
+                cutoff = x;
+                found = true;
+            }
+        }
+        if (!found) cutoff = sp[0];  // never reached: only the maximum survives
+        keep = keep && pr >= cutoff;
+        if (!keep) pr = 0.0f;
+        __builtin_amdgcn_wave_barrier();
+        se[lane] = pr;
+        __builtin_amdgcn_wave_barrier();
+        float total = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 64; j++) total += se[j];  // cut entries add an exact zero
+        if (total > 0.0f) pr = pr / total;
+        __builtin_amdgcn_wave_barrier();
+        se[lane] = pr;
+        __builtin_amdgcn_wave_barrier();
+    }
+    int chosen = V - 1;
+    if (u <= 0.0f) {
+        chosen = 0;
+    } else {
+        float cumulative = 0.0f;
+        bool found = false;
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+            cumulative += se[j];
+            if (!found && j < S && u <= cumulative) {
+                chosen = sidx[j];
+                found = true;
+            }
+        }
+    }
+    return chosen;
+}
+
 constexpr int kOrderedWalkLimit = 2048;  // survivors sorted by index and walked by one lane
 
-__global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams p) {
-    extern __shared__ float lds[];  // [V] logits -> probabilities, then [sort_cap] sort area
+// The pick for sequence b with the row held in `lds` ([V] values then p.sort_cap
+// floats of sort area).  Every thread of the workgroup must call it; all get the
+// chosen id.  coherent: read the logits with device-scope loads (they were
+// written by other workgroups of the same running kernel).
+__device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool coherent) {
     __shared__ float red[kPickThreads / 64];
     __shared__ int redi[kPickThreads / 64];
     __shared__ unsigned hist256[256];
@@ -476,25 +646,44 @@ __global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams
     __shared__ float fshare[2];
     __shared__ int ishare[2];
 
-    const int b = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
+    const int tid = threadIdx.x, nt = blockDim.x;
     const int V = p.V;
     const float* logits = p.logits + static_cast<size_t>(b) * V;
     float* val = lds;
     float* srt = lds + V;
-    int* hist = p.hist + static_cast<size_t>(b) * p.hist_stride;
+    const int* hist = p.hist + static_cast<size_t>(b) * p.hist_stride;
 
     // ---- logits_with_penalty (text_gen.cpp:14-33)
-    for (int i = tid; i < V; i += nt) val[i] = logits[i];
+    if (coherent) {
+        const __amdgpu_buffer_rsrc_t rs = make_buffer(logits, static_cast<unsigned>(V) * 4u);
+        for (int i = 4 * tid; i < V; i += 4 * nt) {
+            const v4i w = coherent_load16(rs, static_cast<unsigned>(i) * 4u);
+            val[i] = __int_as_float(w.x);
+            if (i + 1 < V) val[i + 1] = __int_as_float(w.y);
+            if (i + 2 < V) val[i + 2] = __int_as_float(w.z);
+            if (i + 3 < V) val[i + 3] = __int_as_float(w.w);
+        }
+    } else {
+        for (int i = tid; i < V; i += nt) val[i] = logits[i];
+    }
     const int window = min(kPenaltyWindow, p.n_hist);
-    if (tid < window) win_tok[tid] = hist[p.n_hist - window + tid];
+    if (tid < window) {
+        const int* hp = &hist[p.n_hist - window + tid];
+        win_tok[tid] = coherent ? __hip_atomic_load(hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *hp;
+    }
+    if (p.dbg && threadIdx.x == 0) p.dbg[0] = __builtin_amdgcn_s_memrealtime();
     __syncthreads();
-    if (p.penalty != 1.0f && tid < window) {
-        const int id = win_tok[tid];
-        bool first = true;
-        for (int e = 0; e < tid; e++) first = first && (win_tok[e] != id);
-        if (first) {
-            int count = 0;
-            for (int e = tid; e < window; e++) count += (win_tok[e] == id);
+    if (p.penalty != 1.0f && tid < 64) {
+        // lane e holds window entry e; a token is handled by its first occurrence,
+        // which applies the penalty once per occurrence
+        const int id = tid < window ? win_tok[tid] : -1 - tid;
+        int before = 0, count = 0;
+        for (int e = 0; e < kPenaltyWindow; e++) {
+            const int other = __builtin_amdgcn_readlane(id, e);
+            before += (e < tid && other == id);
+            count += (other == id);
+        }
+        if (tid < window && before == 0) {
             float v = val[id];
             for (int c = 0; c < count; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
             val[id] = v;
@@ -502,6 +691,7 @@ __global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams
     }
     __syncthreads();
 
+    if (p.dbg && threadIdx.x == 0) p.dbg[1] = __builtin_amdgcn_s_memrealtime();
     int chosen;
     if (p.greedy) {
         float best = -INFINITY;
@@ -543,8 +733,44 @@ __global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams
         const float inv_t = 1.0f / p.temperature;
         for (int i = tid; i < V; i += nt) val[i] = val[i] * inv_t;
         __syncthreads();
+        float u;
+        if (p.uniforms) {
+            u = p.uniforms[static_cast<size_t>(b) * p.u_stride + p.pick_idx];
+        } else {
+            const unsigned w = philox4x32_10(static_cast<unsigned>(p.pick_idx) >> 2,
+                                             static_cast<unsigned>(p.pick_idx) & 3u, p.seed_lo,
+                                             p.seed_hi ^ static_cast<unsigned>(b));
+            u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
+        }
+        if (p.dbg && threadIdx.x == 0) p.dbg[2] = __builtin_amdgcn_s_memrealtime();
         if (p.top_k > 0 && p.top_k < V) {
-            const float thr = kth_largest_lds(val, V, p.top_k, hist256, bcast);
+            const float thr = kth_largest_block(val, V, p.top_k, srt, p.sort_cap, hist256, bcast, ishare);
+            if (p.dbg && threadIdx.x == 0) p.dbg[3] = __builtin_amdgcn_s_memrealtime();
+            // Survivors of the cut (ties at the threshold included).  When they fit
+            // one wavefront the rest of the sampler runs there.
+            int* cidx = reinterpret_cast<int*>(srt);
+            if (tid == 0) ishare[1] = 0;
+            __syncthreads();
+            for (int i = tid; i < V; i += nt) {
+                if (val[i] >= thr) {
+                    const int slot = atomicAdd(&ishare[1], 1);
+                    if (slot < 64) cidx[slot] = i;
+                }
+            }
+            __syncthreads();
+            if (p.dbg && threadIdx.x == 0) p.dbg[4] = __builtin_amdgcn_s_memrealtime();
+            const int S0 = ishare[1];
+            if (S0 <= 64 && p.sort_cap >= 512) {
+                if (tid < 64) {
+                    const int c = pick_small_wave(val, cidx, S0, p.top_p, u, V, srt + 64);
+                    if (tid == 0) ishare[0] = c;
+                }
+                __syncthreads();
+                if (p.dbg && threadIdx.x == 0) p.dbg[5] = __builtin_amdgcn_s_memrealtime();
+                const int c = ishare[0];
+                __syncthreads();
+                return c;
+            }
             for (int i = tid; i < V; i += nt)
                 if (val[i] < thr) val[i] = -1e10f;
             __syncthreads();
@@ -610,15 +836,6 @@ __global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams
         }
         __syncthreads();
 
-        float u;
-        if (p.uniforms) {
-            u = p.uniforms[static_cast<size_t>(b) * p.u_stride + p.pick_idx];
-        } else {
-            const unsigned w = philox4x32_10(static_cast<unsigned>(p.pick_idx) >> 2,
-                                             static_cast<unsigned>(p.pick_idx) & 3u, p.seed_lo,
-                                             p.seed_hi ^ static_cast<unsigned>(b));
-            u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
-        }
         const bool renorm = p.top_p < 1.0f;
 
         if (S <= kOrderedWalkLimit && S <= p.sort_cap) {
@@ -704,9 +921,16 @@ __global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams
         __syncthreads();
         chosen = ishare[0];
     }
+    __syncthreads();
+    return chosen;
+}
 
-    if (tid == 0) {
-        hist[p.n_hist] = chosen;
+__global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams p) {
+    extern __shared__ float lds[];
+    const int b = blockIdx.x;
+    const int chosen = pick_lds_body(p, b, lds, false);
+    if (threadIdx.x == 0) {
+        p.hist[static_cast<size_t>(b) * p.hist_stride + p.n_hist] = chosen;  // tokens.push_back(next)
         p.tok[b] = chosen;
     }
 }
