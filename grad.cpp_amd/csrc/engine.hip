@@ -456,6 +456,14 @@ static void launch_gemv(const GemvParams& p, int batch, hipStream_t st) {
 static void launch_attn(const AttnParams& p, int batch, hipStream_t st) {
     const int hs = p.kv.head_size;
     const dim3 grid(p.max_chunks, p.kv.heads, batch);
+    if (hs == 64) {
+        if (p.kv.page_shift >= 5 && p.chunk % 128 == 0)
+            hipLaunchKernelGGL(attn_decode64_kernel<true>, grid, dim3(256), 0, st, p);
+        else
+            hipLaunchKernelGGL(attn_decode64_kernel<false>, grid, dim3(256), 0, st, p);
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
     const size_t lds = (static_cast<size_t>(p.chunk) + 4 * hs + 8) * sizeof(float);
     switch (hs) {
         case 8: hipLaunchKernelGGL(attn_decode_kernel<8>, grid, dim3(256), lds, st, p); break;
@@ -840,11 +848,13 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     HIP_CHECK(hipHostMalloc(&s.host_ids, B * s.hist_stride * sizeof(int)));
     HIP_CHECK(hipHostMalloc(&s.host_err, sizeof(int)));
 
-    // Attention chunking: enough workgroups to cover the GPU, at most 1024
-    // positions per workgroup (their scores live in LDS).
-    int chunk = 64;
-    while (chunk < 1024 && static_cast<long>(B) * sh.heads * ((sh.max_len + chunk - 1) / chunk) > 2048)
-        chunk *= 2;
+    // Attention chunking: a (sequence, head) is split over several workgroups
+    // only while that is needed to cover the GPU (at least ~512 workgroups); a
+    // chunk is at most 1024 positions (the any-head-size kernel keeps its
+    // scores in LDS).
+    int chunk = 1024;
+    while (chunk > 128 && static_cast<long>(B) * sh.heads * ((sh.max_len + chunk - 1) / chunk) < 512)
+        chunk /= 2;
     s.attn_chunk = chunk;
     s.attn_max_chunks = (sh.max_len + chunk - 1) / chunk;
     dev_alloc(s.attn_part, B * sh.heads * s.attn_max_chunks * (sh.head_size() + 2));

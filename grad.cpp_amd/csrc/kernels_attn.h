@@ -25,18 +25,41 @@ struct AttnParams {
     unsigned* tickets;  // [batch][heads], zero between launches
 };
 
-// Merges chunk partials (running max m, sum l, unnormalised acc) of one head.
+// How chunks of one (sequence, head) meet without flushing caches: a chunk writes
+// its partial (running max m, sum l, unnormalised acc) with device-scope stores,
+// waits for them to be acknowledged, then takes a ticket with a device-scope
+// atomic; the chunk that draws the last ticket reads all partials back with
+// device-scope loads and merges them.
+__device__ __forceinline__ void partial_store(float* dst, float v) {
+    __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Every thread of the workgroup calls this after its partial_store calls;
+// returns true in the workgroup that must merge.
+__device__ __forceinline__ bool last_chunk_arrived(unsigned* ticket_ctr, int nchunk, unsigned* lds_slot) {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0)
+        *lds_slot = __hip_atomic_fetch_add(ticket_ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    return *lds_slot == static_cast<unsigned>(nchunk - 1);
+}
+
 __device__ __forceinline__ void attn_merge(const AttnParams& p, int b, int h, int nchunk, int hs) {
     const float* base = p.part + (static_cast<size_t>(b) * p.kv.heads + h) * p.max_chunks * (hs + 2);
+    const __amdgpu_buffer_rsrc_t rs = make_buffer(base, static_cast<unsigned>(nchunk * (hs + 2)) * 4u);
+    auto at = [&](int i) {  // one float through a device-scope load
+        const v4i w = coherent_load16(rs, static_cast<unsigned>(i & ~3) * 4u);
+        return __int_as_float(w[i & 3]);
+    };
     float M = -INFINITY;
-    for (int s = 0; s < nchunk; s++) M = fmaxf(M, base[s * (hs + 2)]);
+    for (int s = 0; s < nchunk; s++) M = fmaxf(M, at(s * (hs + 2)));
     float L = 0.0f;
-    for (int s = 0; s < nchunk; s++) L += base[s * (hs + 2) + 1] * expf(base[s * (hs + 2)] - M);
+    for (int s = 0; s < nchunk; s++) L += at(s * (hs + 2) + 1) * expf(at(s * (hs + 2)) - M);
     const float inv = 1.0f / L;
     for (int j = threadIdx.x; j < hs; j += blockDim.x) {
         float o = 0.0f;
-        for (int s = 0; s < nchunk; s++)
-            o += base[s * (hs + 2) + 2 + j] * expf(base[s * (hs + 2)] - M);
+        for (int s = 0; s < nchunk; s++) o += at(s * (hs + 2) + 2 + j) * expf(at(s * (hs + 2)) - M);
         p.out[static_cast<size_t>(b) * p.d_model + h * hs + j] = o * inv;
     }
 }
@@ -153,22 +176,163 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnParams p) {
     for (int j = tid; j < hs; j += blockDim.x) {
         float o = 0.0f;
         for (int w = 0; w < nred; w++) o += red[w * hs + j];
-        mine[2 + j] = o;
+        partial_store(mine + 2 + j, o);
     }
     if (tid == 0) {
-        mine[0] = m;
-        mine[1] = l;
+        partial_store(mine, m);
+        partial_store(mine + 1, l);
     }
-    // Publish the partial, then take a ticket; the last chunk to arrive merges.
-    __threadfence();
-    __syncthreads();
     __shared__ unsigned ticket;
-    if (tid == 0) ticket = atomicAdd(&p.tickets[b * p.kv.heads + h], 1u);
-    __syncthreads();
-    if (ticket != static_cast<unsigned>(nchunk - 1)) return;
-    __threadfence();
+    if (!last_chunk_arrived(&p.tickets[b * p.kv.heads + h], nchunk, &ticket)) return;
     attn_merge(p, b, h, nchunk, hs);
-    if (tid == 0) p.tickets[b * p.kv.heads + h] = 0u;
+    if (tid == 0) __hip_atomic_store(&p.tickets[b * p.kv.heads + h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace gh
+
+namespace gh {
+
+// ---------------------------------------------------------------------------
+// Head size 64, throughput form: each wavefront owns a contiguous run of
+// positions and walks it 32 positions at a time entirely in registers — 16
+// lanes hold one position's 64 floats, four positions per load instruction,
+// eight K and eight V loads in flight per lane — keeping a running (max, sum,
+// weighted V) that is rescaled when the maximum moves.  The four wavefronts of
+// a workgroup, and the workgroups that share a (sequence, head), are merged the
+// same way.  This is the kernel for many sequences or long contexts, where the
+// cache, not the weights, is most of the bytes of a step.
+
+// Sum over each aligned group of 16 lanes, every lane of the group gets it.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xB1, 0xF>(v, 0.0f);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xF>(v, 0.0f);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xF>(v, 0.0f);  // row_half_mirror
+    v += dpp_move<0x140, 0xF>(v, 0.0f);  // row_mirror
+    return v;
+}
+
+// PAGE32: pages hold at least 32 positions, so an aligned batch of 32 sits in
+// one page and its page number is one scalar lookup.
+template <bool PAGE32>
+__global__ __launch_bounds__(256) void attn_decode64_kernel(const AttnParams p) {
+    constexpr int HS = 64;
+    __shared__ float part[4][68];  // per wavefront: m, l, pad, pad, acc[64]
+    __shared__ unsigned ticket;
+    const int ck = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int ctx = p.st->pos + 1;
+    const int nchunk = (ctx + p.chunk - 1) / p.chunk;
+    if (ck >= nchunk) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane >> 4, dl = lane & 15;
+    const int c0 = ck * p.chunk, c1 = min(ctx, c0 + p.chunk);
+    // positions of the chunk are dealt to the wavefronts in runs that are multiples of 32
+    const int run = ((((c1 - c0) + 3) / 4) + 31) & ~31;
+    const int t0 = c0 + wave * run, t1 = min(c1, t0 + run);
+    const float* pool = p.kv.pool;
+    const float4 q4 = reinterpret_cast<const float4*>(p.q + static_cast<size_t>(b) * p.d_model + h * HS)[dl];
+    const int shift = p.kv.page_shift;
+    const int* table = p.kv.page_table + b * p.kv.pages_per_seq;
+    const size_t head_stride = static_cast<size_t>(HS) << shift;               // floats per (page, K|V, head)
+    const size_t kv_stride = head_stride * p.kv.heads;                         // K -> V within a page
+    const size_t page_stride = 2 * kv_stride;
+    const size_t layer_base = static_cast<size_t>(p.layer) * p.kv.n_pages * page_stride + h * head_stride;
+
+    float m = -INFINITY, lsum = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int tb = t0; tb < t1; tb += 32) {
+        float4 k4[8], v4[8];
+        size_t base = 0;
+        if (PAGE32) base = layer_base + static_cast<size_t>(table[tb >> shift]) * page_stride;
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const int tt = tb + it * 4 + sub;
+            k4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            v4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (tt < t1) {
+                size_t off;
+                if (PAGE32) {
+                    off = base + static_cast<size_t>(tt & ((1 << shift) - 1)) * HS + dl * 4;
+                } else {
+                    off = layer_base + static_cast<size_t>(table[tt >> shift]) * page_stride
+                          + static_cast<size_t>(tt & ((1 << shift) - 1)) * HS + dl * 4;
+                }
+                k4[it] = *reinterpret_cast<const float4*>(pool + off);
+                v4[it] = *reinterpret_cast<const float4*>(pool + off + kv_stride);
+            }
+        }
+        float sc[8];
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const int tt = tb + it * 4 + sub;
+            const float sdot = row16_sum(dot4(q4, k4[it]));
+            sc[it] = tt < t1 ? sdot * p.scale : -INFINITY;
+        }
+        float mb = sc[0];
+#pragma unroll
+        for (int it = 1; it < 8; it++) mb = fmaxf(mb, sc[it]);
+        // the four position groups of the wavefront share one running maximum
+        mb = fmaxf(mb, dpp_move<0x142, 0xA>(mb, mb));
+        mb = fmaxf(mb, dpp_move<0x143, 0xC>(mb, mb));
+        mb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mb), 63));
+        const float mn = fmaxf(m, mb);
+        const float f = expf(m - mn);  // 0 on the first batch
+        lsum *= f;
+        acc.x *= f;
+        acc.y *= f;
+        acc.z *= f;
+        acc.w *= f;
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const float e = expf(sc[it] - mn);  // exp(-inf) = 0 past the end of the run
+            lsum += e;
+            acc.x += e * v4[it].x;
+            acc.y += e * v4[it].y;
+            acc.z += e * v4[it].z;
+            acc.w += e * v4[it].w;
+        }
+        m = mn;
+    }
+    // fold the four position groups (lanes 16 apart hold the same dims)
+    lsum += __shfl_xor(lsum, 16, kWave);
+    lsum += __shfl_xor(lsum, 32, kWave);
+#pragma unroll
+    for (int o = 16; o < 64; o <<= 1) {
+        acc.x += __shfl_xor(acc.x, o, kWave);
+        acc.y += __shfl_xor(acc.y, o, kWave);
+        acc.z += __shfl_xor(acc.z, o, kWave);
+        acc.w += __shfl_xor(acc.w, o, kWave);
+    }
+    if (lane < 16) reinterpret_cast<float4*>(&part[wave][4])[lane] = acc;
+    if (lane == 0) {
+        part[wave][0] = m;
+        part[wave][1] = lsum;
+    }
+    __syncthreads();
+    if (tid >= HS) {
+        if (nchunk == 1) return;
+    }
+    float M = -INFINITY, L = 0.0f, o = 0.0f;
+    if (tid < HS) {
+        for (int w = 0; w < 4; w++) M = fmaxf(M, part[w][0]);
+        for (int w = 0; w < 4; w++) {
+            const float f = expf(part[w][0] - M);  // 0 for a wavefront without positions
+            L += part[w][1] * f;
+            o += part[w][4 + tid] * f;
+        }
+        if (nchunk == 1) {
+            p.out[static_cast<size_t>(b) * p.d_model + h * HS + tid] = o * (1.0f / L);
+            return;
+        }
+        float* mine = p.part + ((static_cast<size_t>(b) * p.kv.heads + h) * p.max_chunks + ck) * (HS + 2);
+        partial_store(mine + 2 + tid, o);
+        if (tid == 0) {
+            partial_store(mine, M);
+            partial_store(mine + 1, L);
+        }
+    }
+    if (!last_chunk_arrived(&p.tickets[b * p.kv.heads + h], nchunk, &ticket)) return;
+    attn_merge(p, b, h, nchunk, HS);
+    if (tid == 0) __hip_atomic_store(&p.tickets[b * p.kv.heads + h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace gh

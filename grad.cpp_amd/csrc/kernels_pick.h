@@ -467,20 +467,9 @@ __device__ inline float kth_largest_block(const float* v, int n, int k, float* w
     work[tid] = mx;
     if (tid == 0) ishare[1] = 0;
     __syncthreads();
-    {
-        // nt is a multiple of 64: reads in groups of 16 keep the LDS pipeline full
-        int rank = 0;
-        for (int j0 = 0; j0 < nt; j0 += 16) {
-            float o[16];
-#pragma unroll
-            for (int q = 0; q < 16; q++) o[q] = work[j0 + q];
-#pragma unroll
-            for (int q = 0; q < 16; q++) rank += (o[q] > mx) || (o[q] == mx && j0 + q < tid);
-        }
-        if (rank == k - 1) bcast[0] = __float_as_uint(mx);
-    }
+    // one maximum per thread: a radix select over them is four short passes
+    const float T = kth_largest_lds(work, nt, k, hist, bcast);
     __syncthreads();
-    const float T = __uint_as_float(bcast[0]);
     float* cand = work + nt;  // [nt + 16]
     for (int i = tid; i < n; i += nt) {
         const float x = v[i];
