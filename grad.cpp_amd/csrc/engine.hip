@@ -484,6 +484,12 @@ template <int PRO, int EPI>
 static int project(Session& s, GemvParams g, hipStream_t st) {
     const int B = s.B;
     if (B >= kMinGemmBatch && gemm_shape_ok(g.K, g.in_stride)) {
+        if (PRO == PRO_RMSNORM) {
+            // the norm rides inside the projection
+            launch_gemm16<EPI, true>(g, B, st);
+            HIP_CHECK(hipGetLastError());
+            return 1;
+        }
         int launches = 1;
         if (PRO != PRO_PLAIN) {
             hipLaunchKernelGGL(norm_rows_kernel, dim3((B + 3) / 4), dim3(256), 0, st, g.in, g.gamma,
@@ -493,7 +499,7 @@ static int project(Session& s, GemvParams g, hipStream_t st) {
             g.in_stride = g.K;
             launches++;
         }
-        launch_gemm_mfma<EPI>(g, B, st);
+        launch_gemm16<EPI, false>(g, B, st);
         HIP_CHECK(hipGetLastError());
         return launches;
     }
