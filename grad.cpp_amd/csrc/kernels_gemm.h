@@ -55,88 +55,155 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict_
 // RMS: the RMSNorm that precedes the projection is folded in.  A holds the raw
 // residual rows; gamma scales A as it is loaded, the row's sum of squares is
 // accumulated from the same fragments, and 1/rms multiplies the finished dot
-// product (layer_norm_row, inference.cpp:33-43, distributes over the sum).
-template <int EPI, bool RMS>
-__global__ __launch_bounds__(256) void gemm16_kernel(const GemvParams p, int M, int m_tiles) {
-    __shared__ float red[4][16 * 16];
-    __shared__ float ssq[4][16];
+// product (layer_norm_row, inference.cpp:33-43, distributes over the sum).//
+// MT x NT: 16-row tiles of A and 16-row tiles of W per workgroup.  Narrow
+// projections run 1 x 1 (most workgroups); wide ones take the whole batch
+// (MT = 4) so each weight row is fetched once, and the widest also several
+// weight tiles per fetch of A (NT = 4).
+template <int EPI, bool RMS, int MT, int NT, int KW>
+__global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int M, int m_groups) {
+    __shared__ float red[KW][MT][NT][16 * 16];
+    __shared__ float ssq[KW][MT][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // id -> (weight tile, row tile): ids with the same id % 8 and consecutive id / 8 share a weight tile
+    // id -> (weight group, row group): ids with the same id % 8 and consecutive id / 8 share weights
     const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-    const int n_tile = xcd + 8 * (slot / m_tiles), m_tile = slot % m_tiles;
-    const int n0 = n_tile * 16, m0 = m_tile * 16;
+    const int n_group = xcd + 8 * (slot / m_groups), m_group = slot % m_groups;
+    const int n0 = n_group * 16 * NT, m0 = m_group * 16 * MT;
     if (n0 >= p.N) return;
-    const int K = p.K, kq = K / 4;
+    const int K = p.K, kq = K / KW;  // this wavefront's share of K
     const int j = lane & 15, g = lane >> 4;
-    const int wrow = min(n0 + j, p.N - 1), arow = min(m0 + j, M - 1);
-    const float* wp = p.W + static_cast<size_t>(wrow) * K + wave * kq + g * 4;
-    const float* ap = p.in + static_cast<size_t>(arow) * p.in_stride + wave * kq + g * 4;
+    const float* wp[NT];
+    const float* ap[MT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+        wp[t] = p.W + static_cast<size_t>(min(n0 + t * 16 + j, p.N - 1)) * K + wave * kq + g * 4;
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+        ap[t] = p.in + static_cast<size_t>(min(m0 + t * 16 + j, M - 1)) * p.in_stride + wave * kq + g * 4;
     const float* gp = RMS ? p.gamma + wave * kq + g * 4 : nullptr;
-    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
-    float ss = 0.0f;
+    v4f acc[MT][NT];
+    float ss[MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        ss[t] = 0.0f;
+#pragma unroll
+        for (int u = 0; u < NT; u++) acc[t][u] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+    // K-steps of loads in flight: as many as ~100 registers of fragments allow
+    constexpr int UNROLL = (MT + NT + 1) <= 3 ? 8 : (MT + NT + 1) <= 6 ? 4 : 2;
 
-    auto step = [&](const float4& a_raw, const float4& b4, const float4& g4) {
-        float4 a4 = a_raw;
-        if (RMS) {
-            ss += dot4(a_raw, a_raw);
-            a4 = make_float4(a_raw.x * g4.x, a_raw.y * g4.y, a_raw.z * g4.z, a_raw.w * g4.w);
+    auto consume = [&](const float4 (&a)[MT], const float4 (&b)[NT], const float4& g4) {
+        float4 as[MT];
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            as[t] = a[t];
+            if (RMS) {
+                ss[t] += dot4(a[t], a[t]);
+                as[t] = make_float4(a[t].x * g4.x, a[t].y * g4.y, a[t].z * g4.z, a[t].w * g4.w);
+            }
         }
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4.x, b4.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4.y, b4.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4.z, b4.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4.w, b4.w, acc, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int u = 0; u < NT; u++) {
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].x, b[u].x, acc[t][u], 0, 0, 0);
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].y, b[u].y, acc[t][u], 0, 0, 0);
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].z, b[u].z, acc[t][u], 0, 0, 0);
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].w, b[u].w, acc[t][u], 0, 0, 0);
+            }
     };
     int k = 0;
-    for (; k + 64 <= kq; k += 64) {
-        float4 a[4], b[4], gm[4];
+    for (; k + 16 * UNROLL <= kq; k += 16 * UNROLL) {
+        float4 a[UNROLL][MT], b[UNROLL][NT], gm[UNROLL];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            b[u] = *reinterpret_cast<const float4*>(wp + k + 16 * u);
-            a[u] = *reinterpret_cast<const float4*>(ap + k + 16 * u);
+        for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) b[u][t] = *reinterpret_cast<const float4*>(wp[t] + k + 16 * u);
+#pragma unroll
+            for (int t = 0; t < MT; t++) a[u][t] = *reinterpret_cast<const float4*>(ap[t] + k + 16 * u);
             gm[u] = RMS ? *reinterpret_cast<const float4*>(gp + k + 16 * u) : make_float4(1.f, 1.f, 1.f, 1.f);
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) step(a[u], b[u], gm[u]);
+        for (int u = 0; u < UNROLL; u++) consume(a[u], b[u], gm[u]);
     }
     for (; k < kq; k += 16) {
-        const float4 b4 = *reinterpret_cast<const float4*>(wp + k);
-        const float4 a4 = *reinterpret_cast<const float4*>(ap + k);
-        const float4 g4 = RMS ? *reinterpret_cast<const float4*>(gp + k) : make_float4(1.f, 1.f, 1.f, 1.f);
-        step(a4, b4, g4);
-    }
+        float4 a[MT], b[NT];
 #pragma unroll
-    for (int r = 0; r < 4; r++) red[wave][(4 * g + r) * 16 + j] = acc[r];
+        for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const float4*>(wp[t] + k);
+#pragma unroll
+        for (int t = 0; t < MT; t++) a[t] = *reinterpret_cast<const float4*>(ap[t] + k);
+        const float4 g4 = RMS ? *reinterpret_cast<const float4*>(gp + k) : make_float4(1.f, 1.f, 1.f, 1.f);
+        consume(a, b, g4);
+    }
+    // Accumulator layout: lane holds column j, rows 4*g + r.
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int u = 0; u < NT; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) red[wave][t][u][(4 * g + r) * 16 + j] = acc[t][u][r];
     if (RMS) {
         // lanes j, j+16, j+32, j+48 hold the same row's partial sums of squares
-        ss += __shfl_xor(ss, 16, kWave);
-        ss += __shfl_xor(ss, 32, kWave);
-        if (lane < 16) ssq[wave][lane] = ss;
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            float v = ss[t];
+            v += __shfl_xor(v, 16, kWave);
+            v += __shfl_xor(v, 32, kWave);
+            if (lane < 16) ssq[wave][t][lane] = v;
+        }
     }
     __syncthreads();
-    if (threadIdx.x < 128) {
-        const int i = threadIdx.x >> 3, jp = (threadIdx.x & 7) * 2;
-        const int m = m0 + i, n = n0 + jp;
-        if (m < M && n < p.N) {
-            const int at = i * 16 + jp;
-            float v0 = (red[0][at] + red[1][at]) + (red[2][at] + red[3][at]);
-            float v1 = (red[0][at + 1] + red[1][at + 1]) + (red[2][at + 1] + red[3][at + 1]);
-            if (RMS) {
-                const float ms = (ssq[0][i] + ssq[1][i]) + (ssq[2][i] + ssq[3][i]);
-                const float r = 1.0f / sqrtf(ms / static_cast<float>(K) + kNormEps);
-                v0 *= r;
-                v1 *= r;
-            }
-            gemv_epilogue<EPI>(p, m, n, v0, v1, n + 1 < p.N);
+    // Column pairs (n, n+1) of one row go through the shared epilogue.
+    for (int e = threadIdx.x; e < MT * NT * 128; e += 64 * KW) {
+        const int tile = e >> 7, rem = e & 127;
+        const int t = tile / NT, u = tile % NT;
+        const int i = rem >> 3, jp = (rem & 7) * 2;
+        const int m = m0 + t * 16 + i, n = n0 + u * 16 + jp;
+        if (m >= M || n >= p.N) continue;
+        const int at = i * 16 + jp;
+        float v0 = 0.0f, v1 = 0.0f;
+#pragma unroll
+        for (int w = 0; w < KW; w++) {
+            v0 += red[w][t][u][at];
+            v1 += red[w][t][u][at + 1];
         }
+        if (RMS) {
+            float ms = 0.0f;
+#pragma unroll
+            for (int w = 0; w < KW; w++) ms += ssq[w][t][i];
+            const float r = 1.0f / sqrtf(ms / static_cast<float>(K) + kNormEps);
+            v0 *= r;
+            v1 *= r;
+        }
+        gemv_epilogue<EPI>(p, m, n, v0, v1, n + 1 < p.N);
     }
 }
 
+template <int EPI, bool RMS, int MT, int NT, int KW>
+inline void launch_gemm16_as(const GemvParams& p, int M, hipStream_t st) {
+    const int m_groups = (M + 16 * MT - 1) / (16 * MT);
+    const int n_groups = (p.N + 16 * NT - 1) / (16 * NT);
+    const int n_groups8 = (n_groups + 7) / 8 * 8;  // whole rounds of the 8 XCDs
+    hipLaunchKernelGGL((gemm16_kernel<EPI, RMS, MT, NT, KW>), dim3(n_groups8 * m_groups), dim3(64 * KW), 0,
+                       st, p, M, m_groups);
+}
+
+// K is split over 8 wavefronts when that leaves each a multiple of 16.
 template <int EPI, bool RMS>
 inline void launch_gemm16(const GemvParams& p, int M, hipStream_t st) {
-    const int m_tiles = (M + 15) / 16;
-    const int n_tiles = (p.N + 15) / 16;
-    const int n_tiles8 = (n_tiles + 7) / 8 * 8;  // whole rounds of the 8 XCDs
-    hipLaunchKernelGGL((gemm16_kernel<EPI, RMS>), dim3(n_tiles8 * m_tiles), dim3(256), 0, st, p, M, m_tiles);
+    const bool k8 = p.K % 128 == 0;
+    if (p.N <= 1024 || M <= 16) {
+        if (k8) launch_gemm16_as<EPI, RMS, 1, 1, 8>(p, M, st);
+        else launch_gemm16_as<EPI, RMS, 1, 1, 4>(p, M, st);
+    } else if (M <= 32) {
+        if (k8) launch_gemm16_as<EPI, RMS, 2, 1, 8>(p, M, st);
+        else launch_gemm16_as<EPI, RMS, 2, 1, 4>(p, M, st);
+    } else if (p.N <= 8192) {
+        if (k8) launch_gemm16_as<EPI, RMS, 4, 1, 8>(p, M, st);
+        else launch_gemm16_as<EPI, RMS, 4, 1, 4>(p, M, st);
+    } else {
+        launch_gemm16_as<EPI, RMS, 4, 2, 4>(p, M, st);
+    }
 }
 
 // The MFMA path needs K % 64 == 0 and 16-byte aligned rows; other shapes walk
