@@ -1,0 +1,232 @@
+// gradhip.hpp — header-only C++20 adapter over the C ABI of gradhip.h.
+//
+// It gives callers written against grad.cpp's generation API the same class
+// names, signatures, ownership rules and exception types, so that a caller like
+// src/cli/generate.cpp or src/cli/chat.cpp changes one include and one
+// namespace:
+//
+//     grad::GPTModel::load            -> gradhip::GPTModel::load      (gpt_model.h:87)
+//     grad::InferenceSession          -> gradhip::InferenceSession    (inference.h:16-29)
+//     grad::TextGen                   -> gradhip::TextGen             (text_gen.h:12-38)
+//     grad::Tokenizer (decode only)   -> gradhip::Tokenizer           (tokenizer.h:20-43)
+//
+// The model lives on the GPU; there is no CPU path behind these classes.
+#pragma once
+
+#include "gradhip.h"
+
+#include <cstdint>
+#include <functional>
+#include <optional>
+#include <random>
+#include <span>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace gradhip {
+
+// Maps a C-ABI status to the exception grad.cpp throws at the same point.
+inline void check(gh_status st) {
+    if (st == GH_OK) return;
+    const std::string msg = gh_last_error();
+    switch (st) {
+        case GH_ERR_OUT_OF_RANGE: throw std::out_of_range(msg);
+        case GH_ERR_INVALID_ARGUMENT: throw std::invalid_argument(msg);
+        default: throw std::runtime_error(msg);
+    }
+}
+
+enum class GPTArch { GPT2 = 0, Modern = 1 };            // gpt_model.h:31
+enum class TokenizerKind { BpeV1 = 1, ByteBpe = 2 };    // grad/tokenizer/fingerprint.h
+
+struct TokenizerFingerprint {
+    TokenizerKind kind;
+    std::uint64_t hash;
+    bool operator==(const TokenizerFingerprint&) const = default;
+};
+
+// The part of grad::Tokenizer the generation path uses (text_gen.cpp:122-125).
+class Tokenizer {
+public:
+    virtual ~Tokenizer() = default;
+    [[nodiscard]] virtual std::string decode(std::span<const int> ids) const = 0;
+};
+
+class GPTModel {
+public:
+    // Throws std::runtime_error with GPTModel::load's messages (gpt_model.cpp:383-525).
+    [[nodiscard]] static GPTModel load(const std::string& filepath) {
+        gh_model* m = nullptr;
+        check(gh_model_load(filepath.c_str(), &m));
+        return GPTModel(m);
+    }
+
+    // Checkpoint-order host tensors, (in, out) row-major (gpt_model.cpp:318-355).
+    [[nodiscard]] static GPTModel from_host(const gh_config& cfg, const std::vector<const float*>& tensors) {
+        gh_model* m = nullptr;
+        check(gh_model_from_host(&cfg, tensors.data(), static_cast<int32_t>(tensors.size()), &m));
+        return GPTModel(m);
+    }
+
+    // GPTModel::save (gpt_model.cpp:292-381); false when the file cannot be written.
+    [[nodiscard]] bool save(const std::string& filepath, bool /*quiet*/ = false) const {
+        return gh_model_save(m_, filepath.c_str()) == GH_OK;
+    }
+
+    int getVocabSize() const { return cfg_.vocab; }
+    int getDModel() const { return cfg_.d_model; }
+    int getNumLayers() const { return cfg_.layers; }
+    int getNumHeads() const { return cfg_.heads; }
+    int getMaxLen() const { return cfg_.max_len; }
+    GPTArch getArch() const { return static_cast<GPTArch>(cfg_.arch); }
+    std::optional<TokenizerFingerprint> getTokenizerFingerprint() const {
+        if (!cfg_.has_fingerprint) return std::nullopt;
+        return TokenizerFingerprint{static_cast<TokenizerKind>(cfg_.tokenizer_kind), cfg_.tokenizer_hash};
+    }
+
+    GPTModel(const GPTModel&) = delete;
+    GPTModel& operator=(const GPTModel&) = delete;
+    GPTModel(GPTModel&& o) noexcept : m_(std::exchange(o.m_, nullptr)), cfg_(o.cfg_) {}
+    GPTModel& operator=(GPTModel&& o) noexcept {
+        if (this != &o) {
+            gh_model_free(m_);
+            m_ = std::exchange(o.m_, nullptr);
+            cfg_ = o.cfg_;
+        }
+        return *this;
+    }
+    ~GPTModel() { gh_model_free(m_); }
+
+    gh_model* handle() const { return m_; }
+
+private:
+    explicit GPTModel(gh_model* m) : m_(m) { check(gh_model_get_config(m_, &cfg_)); }
+    gh_model* m_ = nullptr;
+    gh_config cfg_{};
+};
+
+// Incremental decoding with a KV cache (inference.h:16-29).  The model must
+// outlive the session; the pointer step() returns is valid until the next step().
+class InferenceSession {
+public:
+    explicit InferenceSession(const GPTModel& model) : model_(model) {
+        gh_session_opts o{};
+        o.batch = 1;
+        check(gh_session_create(model.handle(), &o, &s_));
+    }
+    InferenceSession(const InferenceSession&) = delete;
+    InferenceSession& operator=(const InferenceSession&) = delete;
+    ~InferenceSession() { gh_session_free(s_); }
+
+    // Throws std::runtime_error("InferenceSession: context exceeds max_len") or
+    // std::out_of_range("InferenceSession: token id out of vocab range") (inference.cpp:151-156).
+    [[nodiscard]] const float* step(int token_id) {
+        const int32_t id = token_id;
+        check(gh_session_step(s_, &id, nullptr));
+        const float* logits = nullptr;
+        check(gh_session_logits(s_, &logits));
+        return logits;
+    }
+
+    int position() const { return gh_session_position(s_); }
+    int capacity() const { return gh_session_capacity(s_); }
+    int vocabSize() const { return gh_session_vocab(s_); }
+
+    gh_session* handle() const { return s_; }
+
+private:
+    const GPTModel& model_;
+    gh_session* s_ = nullptr;
+};
+
+class TextGen {
+public:
+    // Without a tokenizer, each token id is printed as the byte it equals (text_gen.cpp:127-132).
+    explicit TextGen(const GPTModel& model, const Tokenizer* tok = nullptr) : model_(model), tokenizer_(tok) {}
+
+    // grad.cpp draws from a process-wide std::mt19937 seeded by std::random_device
+    // (text_gen.cpp:195-197), so its streams are not repeatable.  Here the draws
+    // come from a counter-based generator on the GPU whose seed is random unless fixed.
+    void set_seed(std::uint64_t seed) { seed_ = seed; }
+
+    std::string generate_greedy(const std::vector<int>& prompt_tokens, int max_tokens = 50,
+                                float repetition_penalty = 1.2f) {
+        gh_sampling o{1.0f, 0, 1.0f, repetition_penalty, 1};
+        return tokens_to_string(run(prompt_tokens, max_tokens, o));
+    }
+
+    std::string generate_sample(const std::vector<int>& prompt_tokens, float temperature = 1.0f,
+                                int max_tokens = 50, float repetition_penalty = 1.2f, int top_k = 0,
+                                float top_p = 1.0f) {
+        gh_sampling o{temperature, top_k, top_p, repetition_penalty, 0};
+        return tokens_to_string(run(prompt_tokens, max_tokens, o));
+    }
+
+    // Invokes on_text with each token's text as soon as it is sampled; returns
+    // the number of tokens generated (text_gen.cpp:93-120).
+    int generate_stream(const std::vector<int>& prompt_tokens,
+                        const std::function<void(const std::string&)>& on_text, float temperature = 1.0f,
+                        int max_tokens = 50, float repetition_penalty = 1.2f, int top_k = 0,
+                        float top_p = 1.0f) {
+        if (prompt_tokens.empty()) return 0;
+        InferenceSession session(model_);
+        std::vector<int32_t> ids(prompt_tokens.begin(), prompt_tokens.end());
+        check(gh_session_prefill(session.handle(), ids.data(), static_cast<int32_t>(ids.size()), nullptr));
+        gh_sampling o{temperature, top_k, top_p, repetition_penalty, 0};
+        const std::uint64_t seed = next_seed();
+        int generated = 0;
+        for (int i = 0; i < max_tokens; i++) {
+            // a pick made with the context already full is pushed but not stepped,
+            // and ends the loop (text_gen.cpp:116)
+            const bool full = session.position() >= session.capacity();
+            int32_t tok = 0, made = 0;
+            check(gh_session_decode(session.handle(), 1, &o, nullptr, seed, &tok, &made));
+            if (made == 0) break;
+            generated++;
+            on_text(tokens_to_string({static_cast<int>(tok)}));
+            if (full) break;
+        }
+        return generated;
+    }
+
+    // The token ids of the last generate_greedy / generate_sample call.
+    const std::vector<int>& last_tokens() const { return last_; }
+
+private:
+    std::vector<int> run(const std::vector<int>& prompt, int max_tokens, const gh_sampling& o) {
+        last_.clear();
+        if (prompt.empty()) return {};  // text_gen.cpp:40
+        InferenceSession session(model_);
+        std::vector<int32_t> ids(prompt.begin(), prompt.end());
+        const int cap = static_cast<int>(ids.size()) + (max_tokens > 0 ? max_tokens : 0);
+        std::vector<int32_t> out(static_cast<size_t>(cap));
+        int32_t n = 0;
+        check(gh_session_generate(session.handle(), ids.data(), static_cast<int32_t>(ids.size()), max_tokens,
+                                  &o, nullptr, next_seed(), out.data(), &n, nullptr, nullptr));
+        last_.assign(out.begin(), out.begin() + n);
+        return last_;
+    }
+
+    std::string tokens_to_string(const std::vector<int>& tokens) const {
+        if (tokenizer_ != nullptr) return tokenizer_->decode(tokens);
+        std::string result;
+        result.reserve(tokens.size());
+        for (int token : tokens) result += static_cast<char>(token);
+        return result;
+    }
+
+    std::uint64_t next_seed() {
+        if (seed_) return *seed_;
+        std::random_device rd;
+        return (static_cast<std::uint64_t>(rd()) << 32) | rd();
+    }
+
+    const GPTModel& model_;
+    const Tokenizer* tokenizer_;
+    std::optional<std::uint64_t> seed_;
+    std::vector<int> last_;
+};
+
+}  // namespace gradhip

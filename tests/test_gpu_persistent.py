@@ -1,0 +1,98 @@
+"""The persistent batch-1 engine (one kernel launch per run of steps) against the
+CPU oracle and against the one-kernel-per-op engine, on shapes it has kernels
+for: head size 64, d_model 512/768, GPT-2 and Llama blocks."""
+import numpy as np
+import pytest
+
+import gradhip as G
+import oracle_lib as O
+from gradhip import synth
+from helpers import assert_logits_close, check_greedy_stream, check_sampled_stream, make_pair
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {
+    "gpt2-d512": synth.Config(synth.ARCH_GPT2, 1000, 512, 2, 8, 64),
+    "gpt2-d768": synth.Config(synth.ARCH_GPT2, 700, 768, 2, 12, 72),
+    "llama-d768": synth.Config(synth.ARCH_MODERN, 1200, 768, 2, 12, 96),
+}
+
+
+@pytest.fixture(scope="module")
+def models():
+    out = {}
+    for name, cfg in SHAPES.items():
+        W, om = make_pair(cfg, 21, std=0.05, norm_noise=0.1)
+        out[name] = (cfg, W, om, G.Model.from_tensors(cfg, W))
+    return out
+
+
+@pytest.mark.parametrize("name", sorted(SHAPES))
+def test_auto_engine_is_persistent_and_steps_match(models, name):
+    cfg, W, om, gm = models[name]
+    auto = G.Session(gm)  # picks the persistent engine for these shapes
+    forced = G.Session(gm, engine=G.ENGINE_PERSISTENT, shuffle_pages=True, page_tokens=8)
+    graph = G.Session(gm, engine=G.ENGINE_GRAPH)
+    osess = O.Session(om)
+    for t in synth.uniform_tokens(cfg.max_len, cfg.vocab, 5):
+        ref = osess.step(t)
+        a = auto.step([t])[0]
+        assert_logits_close(a, ref, 1e-4, f"{name} step {osess.position}")
+        assert np.array_equal(a, forced.step([t])[0])      # page placement does not matter
+        assert_logits_close(graph.step([t])[0], a, 2e-5)    # two engines, same numbers up to sum order
+    with pytest.raises(RuntimeError, match="InferenceSession: context exceeds max_len"):
+        auto.step([1])
+    for layer in range(cfg.layers):
+        for pos in (0, cfg.max_len - 1):
+            assert np.abs(forced.read_kv(0, layer, 0, pos) - osess.k_row(layer, pos)).max() < 2e-5
+            assert np.abs(forced.read_kv(0, layer, 1, pos) - osess.v_row(layer, pos)).max() < 2e-5
+
+
+@pytest.mark.parametrize("name", sorted(SHAPES))
+def test_generate_loops(models, name):
+    cfg, W, om, gm = models[name]
+    prompt = synth.uniform_tokens(7, cfg.vocab, 6)
+    prompt[4] = prompt[2]
+    n = cfg.max_len - 7 + 5   # runs into the capacity rule
+    u = synth.uniforms(n, 9)
+    s = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    for penalty in (1.0, 1.2):
+        ref, rsl = O.generate_greedy(om, prompt, n, penalty, want_logits=True)
+        got, gsl = s.generate(prompt, n, G.sampling(greedy=True, repetition_penalty=penalty), want_logits=True)
+        check_greedy_stream(got[0], ref, rsl, 7, f"{name} greedy {penalty}")
+        assert got.shape[1] == len(ref) == cfg.max_len + 1 and len(gsl) == len(rsl) == cfg.max_len
+    for opts in ((0.8, 40, 0.9, 1.1), (1.0, 0, 1.0, 1.2), (0.7, 0, 0.8, 1.0), (1.3, 5, 1.0, 1.3)):
+        T, k, p, pen = opts
+        ref, rsl = O.generate_sample(om, prompt, u, T, n, pen, k, p, want_logits=True)
+        got = s.generate(prompt, n, G.sampling(T, k, p, pen), uniforms=u)
+        check_sampled_stream(got[0], ref, rsl, 7, u, opts, f"{name} {opts}")
+        assert np.array_equal(s.generate(prompt, n, G.sampling(T, k, p, pen), seed=9), got)
+
+
+def test_prefill_then_decode_continues_the_context(models):
+    cfg, W, om, gm = models["llama-d768"]
+    prompt = synth.uniform_tokens(20, cfg.vocab, 7)
+    opt = G.sampling(0.9, 10, 0.95, 1.15)
+    u = synth.uniforms(30, 8)
+    whole = G.Session(gm, engine=G.ENGINE_PERSISTENT).generate(prompt, 30, opt, uniforms=u)[0]
+    s = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    s.prefill(prompt[:11])
+    s.prefill(prompt[11:])
+    a = s.decode(12, opt, uniforms=u[:12])[0]
+    b = s.decode(18, opt, uniforms=u[12:])[0]
+    assert np.concatenate([prompt, a, b]).tolist() == whole.tolist()
+    # and the single-pick API agrees with the loop
+    t = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    for tok in prompt:
+        t.step([tok])
+    assert int(t.pick(opt, uniforms=[u[0]])[0]) == int(whole[20])
+
+
+def test_unsupported_shapes_fall_back_or_refuse(models):
+    cfg = synth.Config(synth.ARCH_MODERN, 301, 128, 2, 2, 40)
+    gm = G.Model.from_tensors(cfg, synth.make_weights(cfg, 1))
+    G.Session(gm)  # auto: falls back to the graph engine
+    with pytest.raises(ValueError, match="persistent engine"):
+        G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    with pytest.raises(ValueError, match="persistent engine"):
+        G.Session(models["llama-d768"][3], batch=2, engine=G.ENGINE_PERSISTENT)
