@@ -101,7 +101,21 @@ def main():
     ap.add_argument("--engine", default="auto", choices=["auto", "graph", "eager", "persistent"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-batch64", action="store_true", help="skip the batch-64 leg")
+    ap.add_argument("--only-batch64", action="store_true",
+                    help="run only the batch-64 leg and print its object (for profiling that leg alone)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run a 1 GiB device-to-device copy three times (calibrates rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters against a kernel of known traffic) and exit")
     a = ap.parse_args()
+    if a.copy_probe:
+        import torch
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes_read": 1 << 30, "copy_probe_bytes_written": 1 << 30}))
+        return
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (sequences shard across GPUs with no "
                  "exchange; see DESIGN.md); run with --gpus 1")
@@ -118,6 +132,12 @@ def main():
     opts = (0.8, 40, 0.9, 1.1)
     sample = G.sampling(*opts)
 
+    if a.only_batch64:
+        greedy = G.sampling(greedy=True, repetition_penalty=1.0)
+        r64 = run_decode(G, synth, gm, cfg, 64, 128, 128, 16, greedy, 2003, engine)
+        print(json.dumps({"workload": "c3", "value": round(64 * r64["steps"] / r64["wall_s"], 1), "unit": "tok/s",
+                          "us_per_step_gpu": round(r64["gpu_ms"] * 1e3 / r64["steps"], 2)}), flush=True)
+        return
     r1 = run_decode(G, synth, gm, cfg, 1, 32, a.steps, a.warmup, sample, 2002, engine)
     tok_s = r1["steps"] / r1["wall_s"]
     step_us = r1["gpu_ms"] * 1e3 / r1["steps"]

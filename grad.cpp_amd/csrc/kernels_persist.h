@@ -281,11 +281,12 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     float* vin = lds + D;                 // [max(D, F)] attention output / FFN hidden
     float* ascr = vin + (F > D ? F : D);  // attention scratch: q, k, v of the head + wave partials
     int* ptab = reinterpret_cast<int*>(ascr + 192 + kPersistWaves * 68);  // [pages_per_seq]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, wave = tid >> 6;
+    int lane = tid & 63;
     const int wg = blockIdx.x, G = gridDim.x;
     const int V = p.V, L = p.L, H = p.H;
     const int stride = G * kPersistWaves;  // wavefronts in the grid
-    const int first = wg + G * wave;       // item i of a phase goes to workgroup i % G
+    int first = wg + G * wave;             // item i of a phase goes to workgroup i % G
     int i_pick = 0;
     unsigned arrive_gen = p.arrive_base;
     int n_stamp = 0;
@@ -318,9 +319,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     }
 
     constexpr int NQKV = 3 * D / 2;  // phase A items: pairs of rows
-    const bool has_qkv = first < NQKV;
+    const bool has_qkv = wg + G * wave < NQKV;
 
     for (int s = 0; s < p.n_steps; s++) {
+        asm volatile("" : "+v"(lane), "+v"(first));  // as in the layer loop below
         const int pos = p.pos0 + s;
         const unsigned sb = (p.epoch + 1u + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1);
         auto tag_of = [&](int layer, int ph) {
@@ -356,6 +358,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
 
         for (int l = 0; l < L; l++) {
             const LayerPtrs w = p.layers[l];
+            // Keep the compiler from hoisting every lane- and item-derived address of
+            // every phase out of the layer loop (they would not fit in registers and
+            // would be spilled to scratch memory): re-derive them per layer.
+            asm volatile("" : "+v"(lane), "+v"(first));
 
             // ===== phase A: norm1 + QKV (+bias, RoPE) -> q / new k / new v cells and the cache
             for (int item = first; item < NQKV; ) {
