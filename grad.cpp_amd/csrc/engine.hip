@@ -335,6 +335,7 @@ struct Session {
     int sort_cap = 0;
     int pick_lds_floats = 0;  // > 0: the LDS-resident pick kernel fits (vocab + sort area)
     bool pick_global_scratch = false;
+    bool use_prompt_pass = true;
     int launches_per_step = 0;
 
     hipStream_t stream = nullptr;
@@ -359,6 +360,10 @@ struct Session {
     size_t uniforms_cap = 0;
     float* logit_log = nullptr;  // per-step logits for gh_session_generate
     size_t logit_log_cap = 0;
+
+    // prompt pass (all prompt tokens at once): row-major [rows][width] activations
+    float *pp_x = nullptr, *pp_q = nullptr, *pp_attn = nullptr, *pp_norm = nullptr, *pp_hidden = nullptr;
+    size_t pp_rows = 0;
 
     // persistent engine
     Cell* cells = nullptr;  // xa, xb, q, kn, vn, at (d each), hid (F), token (1)
@@ -409,7 +414,9 @@ struct Session {
                         static_cast<void*>(tok), static_cast<void*>(hist), static_cast<void*>(st),
                         static_cast<void*>(err), static_cast<void*>(uniforms),
                         static_cast<void*>(logit_log), static_cast<void*>(cells),
-                        static_cast<void*>(ctl)})
+                        static_cast<void*>(ctl), static_cast<void*>(pp_x), static_cast<void*>(pp_q),
+                        static_cast<void*>(pp_attn), static_cast<void*>(pp_norm),
+                        static_cast<void*>(pp_hidden)})
             if (p) (void)hipFree(p);
         if (host_logits) (void)hipHostFree(host_logits);
         if (host_ids) (void)hipHostFree(host_ids);
@@ -507,6 +514,26 @@ static int project(Session& s, GemvParams g, hipStream_t st) {
     return 1;
 }
 
+// final norm -> logits = h @ E^T (inference.cpp:251-254) from the rows in s.x
+static int enqueue_logits(Session& s) {
+    const Model& m = *s.m;
+    const Shape& sh = m.shape;
+    const bool modern = sh.modern();
+    GemvParams g{};
+    g.W = m.E;
+    g.bias = nullptr;
+    g.N = sh.vocab;
+    g.K = sh.d_model;
+    g.in = s.x;
+    g.in_stride = sh.d_model;
+    g.gamma = m.gf;
+    g.beta = m.bf;
+    g.out = s.logits;
+    g.out_stride = sh.vocab;
+    return modern ? project<PRO_RMSNORM, EPI_STORE>(s, g, s.stream)
+                  : project<PRO_LAYERNORM, EPI_STORE>(s, g, s.stream);
+}
+
 // One InferenceSession::step for every sequence (inference.cpp:150-258),
 // enqueued on the session stream.  Returns the number of launches.
 static int enqueue_step(Session& s) {
@@ -602,20 +629,7 @@ static int enqueue_step(Session& s) {
         launches += project<PRO_PLAIN, EPI_RESID>(s, g, st);
     }
 
-    // final norm -> logits = h @ E^T (inference.cpp:251-254)
-    GemvParams g{};
-    g.W = m.E;
-    g.bias = nullptr;
-    g.N = V;
-    g.K = d;
-    g.in = s.x;
-    g.in_stride = d;
-    g.gamma = m.gf;
-    g.beta = m.bf;
-    g.out = s.logits;
-    g.out_stride = V;
-    launches += modern ? project<PRO_RMSNORM, EPI_STORE>(s, g, st)
-                       : project<PRO_LAYERNORM, EPI_STORE>(s, g, st);
+    launches += enqueue_logits(s);
 
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, st, s.st);
     HIP_CHECK(hipGetLastError());
@@ -885,6 +899,7 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     size_t v2 = 1024;
     while (v2 < V) v2 *= 2;
     s.pick_global_scratch = (o.flags & GH_FLAG_PICK_GLOBAL_SCRATCH) != 0;
+    s.use_prompt_pass = (o.flags & GH_FLAG_STEPWISE_PROMPT) == 0;
     if (!s.pick_global_scratch && (V + v2) * sizeof(float) + reserve <= static_cast<size_t>(lds_bytes)) {
         s.pick_lds_floats = static_cast<int>(V + v2);
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(pick_lds_kernel),
@@ -1006,10 +1021,161 @@ static void check_pick_error(Session& s) {
     }
 }
 
+// ---- prompt pass: every prompt token of every sequence through each layer at once
+
+constexpr int kPromptPassMin = 8;         // shorter prompts go token by token
+constexpr size_t kPromptPassRows = 32768; // rows per pass; longer prompts run in slices
+
+static bool prompt_pass_ok(const Session& s, int len) {
+    const Shape& sh = s.m->shape;
+    return len >= kPromptPassMin && sh.head_size() == 64 && sh.d_model % 128 == 0 && sh.d_ff() % 128 == 0;
+}
+
+// One projection over M rows (norm folded in for RMSNorm, a norm kernel for LayerNorm).
+template <int PRO, int EPI>
+static void project_rows(Session& s, GemvParams g, int M) {
+    hipStream_t st = s.stream;
+    if (PRO == PRO_RMSNORM) {
+        launch_gemm16<EPI, true>(g, M, st);
+    } else {
+        if (PRO == PRO_LAYERNORM) {
+            hipLaunchKernelGGL(norm_rows_kernel, dim3((M + 3) / 4), dim3(256), 0, st, g.in, g.gamma, g.beta,
+                               s.pp_norm, M, g.K, static_cast<int>(PRO));
+            HIP_CHECK(hipGetLastError());
+            g.in = s.pp_norm;
+            g.in_stride = g.K;
+        }
+        launch_gemm16<EPI, false>(g, M, st);
+    }
+    HIP_CHECK(hipGetLastError());
+}
+
+// Tokens hist[n_hist .. n_hist + len) of every sequence, positions pos .. pos + len.
+// Equivalent to len step() calls (text_gen.cpp:44-46); only the last logits are formed.
+static void prompt_pass(Session& s, int len) {
+    const Model& m = *s.m;
+    const Shape& sh = m.shape;
+    const int d = sh.d_model, F = sh.d_ff(), B = s.B;
+    const bool modern = sh.modern();
+    hipStream_t st = s.stream;
+    const int slice = static_cast<int>(std::max<size_t>(1, std::min<size_t>(len, kPromptPassRows / B)));
+    const size_t rows_cap = static_cast<size_t>(slice) * B;
+    if (s.pp_rows < rows_cap) {
+        for (float** b : {&s.pp_x, &s.pp_q, &s.pp_attn, &s.pp_norm, &s.pp_hidden}) {
+            if (*b) HIP_CHECK(hipFree(*b));
+            *b = nullptr;
+        }
+        dev_alloc(s.pp_x, rows_cap * d);
+        dev_alloc(s.pp_q, rows_cap * d);
+        dev_alloc(s.pp_attn, rows_cap * d);
+        dev_alloc(s.pp_norm, rows_cap * d);
+        dev_alloc(s.pp_hidden, rows_cap * F);
+        s.pp_rows = rows_cap;
+    }
+    for (int t0 = 0; t0 < len; t0 += slice) {
+        const int n = std::min(slice, len - t0);
+        const int M = n * B;
+        const int pos_base = s.pos + t0;
+        hipLaunchKernelGGL(embed_rows_kernel, dim3((d + 255) / 256, M), dim3(256), 0, st, m.E, m.P, s.hist,
+                           s.hist_stride, s.n_hist + t0, n, pos_base, s.pp_x, d);
+        HIP_CHECK(hipGetLastError());
+        for (int l = 0; l < sh.layers; l++) {
+            const LayerWeights& w = m.layers[l];
+            GemvParams g{};
+            g.kv = kv_layout(s);
+            g.layer = l;
+            g.d_model = d;
+            g.st = s.st;
+            g.rows_per_seq = n;
+            g.pos_base = pos_base;
+            g.W = w.wqkv;
+            g.bias = w.bqkv;
+            g.N = 3 * d;
+            g.K = d;
+            g.in = s.pp_x;
+            g.in_stride = d;
+            g.gamma = w.g1;
+            g.beta = w.be1;
+            g.out = s.pp_q;
+            g.out_stride = d;
+            g.rope = modern;
+            g.rope_cos = m.rope_cos;
+            g.rope_sin = m.rope_sin;
+            if (modern) project_rows<PRO_RMSNORM, EPI_QKV>(s, g, M);
+            else project_rows<PRO_LAYERNORM, EPI_QKV>(s, g, M);
+
+            PrefillAttnParams a{};
+            a.q = s.pp_q;
+            a.out = s.pp_attn;
+            a.kv = g.kv;
+            a.layer = l;
+            a.d_model = d;
+            a.len = n;
+            a.pos_base = pos_base;
+            a.scale = 1.0f / std::sqrt(static_cast<float>(sh.head_size()));
+            hipLaunchKernelGGL(attn_prefill64_kernel, dim3((n + 63) / 64, sh.heads, B), dim3(256), 0, st, a);
+            HIP_CHECK(hipGetLastError());
+
+            g.W = w.wo;
+            g.bias = w.bo;
+            g.N = d;
+            g.K = d;
+            g.in = s.pp_attn;
+            g.in_stride = d;
+            g.out = s.pp_x;
+            g.out_stride = d;
+            project_rows<PRO_PLAIN, EPI_RESID>(s, g, M);
+
+            g.in = s.pp_x;
+            g.in_stride = d;
+            g.gamma = w.g2;
+            g.beta = w.be2;
+            g.out = s.pp_hidden;
+            g.out_stride = F;
+            g.W = w.w1;
+            g.K = d;
+            if (modern) {
+                g.bias = nullptr;
+                g.N = 2 * F;
+                project_rows<PRO_RMSNORM, EPI_SWIGLU>(s, g, M);
+            } else {
+                g.bias = w.b1;
+                g.N = F;
+                project_rows<PRO_LAYERNORM, EPI_GELU>(s, g, M);
+            }
+            g.W = w.w2;
+            g.bias = modern ? nullptr : w.b2;
+            g.N = d;
+            g.K = F;
+            g.in = s.pp_hidden;
+            g.in_stride = F;
+            g.out = s.pp_x;
+            g.out_stride = d;
+            project_rows<PRO_PLAIN, EPI_RESID>(s, g, M);
+        }
+        if (t0 + n == len) {
+            hipLaunchKernelGGL(take_last_rows_kernel, dim3((d + 255) / 256, B), dim3(256), 0, st, s.pp_x, n,
+                               s.x, d);
+            HIP_CHECK(hipGetLastError());
+        }
+    }
+    s.pos += len;
+    s.n_hist += len;
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, st, s.st, s.pos, s.n_hist, s.picks);
+    HIP_CHECK(hipGetLastError());
+    // logits of the last position, through the decode-size projection
+    enqueue_logits(s);
+}
+
 // Steps through `len` tokens already staged in the history at n_hist.. (the
 // prompt loop of text_gen.cpp:44-46).  log: per-step logits destination or null.
 static void run_prompt(Session& s, int len, float* log, size_t* steps_logged) {
     const size_t BV = static_cast<size_t>(s.B) * s.m->shape.vocab;
+    if (!log && s.use_prompt_pass && prompt_pass_ok(s, len)) {
+        prompt_pass(s, len);
+        if (steps_logged) *steps_logged += len;
+        return;
+    }
     if (s.engine == GH_ENGINE_PERSISTENT) {
         persist_run(s, len, len, 0, false, nullptr, nullptr, 0, 0,
                     log ? log + *steps_logged * BV : nullptr);

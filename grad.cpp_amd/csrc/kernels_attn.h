@@ -335,4 +335,129 @@ __global__ __launch_bounds__(256) void attn_decode64_kernel(const AttnParams p) 
     if (tid == 0) __hip_atomic_store(&p.tickets[b * p.kv.heads + h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---------------------------------------------------------------------------
+// Prompt pass: causal attention of every new position at once (head size 64).
+// It must give what the per-token loop gives (text_gen.cpp:44-46 stepping
+// inference.cpp:211-225): query t of a sequence sees the cache up to its own
+// position, which the QKV projection of this pass has already written.
+//
+// One workgroup = 64 queries of one (sequence, head).  Keys and values come
+// through LDS in tiles of 64 positions; four threads share a query, each takes
+// every fourth key of a tile and keeps its own running softmax, and the four
+// are merged with quad permutations at the end.
+struct PrefillAttnParams {
+    const float* q;  // [batch * len][d_model], rotated
+    float* out;      // [batch * len][d_model]
+    KvLayout kv;
+    int layer, d_model, len, pos_base;
+    float scale;
+};
+
+__global__ __launch_bounds__(256) void attn_prefill64_kernel(const PrefillAttnParams p) {
+    constexpr int HS = 64, TILE = 64, LD = HS + 4;  // padded rows: the 4 keys of a quad hit different banks
+    __shared__ float Ks[TILE * LD];
+    __shared__ float Vs[TILE * LD];
+    const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, qi = tid >> 2, c = tid & 3;
+    const int t = qb * TILE + qi;                 // this thread's query (token index in the pass)
+    const bool live = t < p.len;
+    const int my_pos = p.pos_base + min(t, p.len - 1);
+    const int last_pos = p.pos_base + min(p.len, qb * TILE + TILE) - 1;  // last key any query here needs
+    float4 q4[16];
+    {
+        const float* qr = p.q + (static_cast<size_t>(b) * p.len + min(t, p.len - 1)) * p.d_model + h * HS;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float4 v = reinterpret_cast<const float4*>(qr)[i];
+            q4[i] = make_float4(v.x * p.scale, v.y * p.scale, v.z * p.scale, v.w * p.scale);
+        }
+    }
+    float m = -INFINITY, l = 0.0f;
+    float4 o4[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) o4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+    for (int k0 = 0; k0 <= last_pos; k0 += TILE) {
+        __syncthreads();
+        // stage the tile: 64 rows of 16 float4 for K and for V, 4 + 4 loads per thread
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int e = tid + r * 256, row = e >> 4, col = e & 15;
+            const int kp = k0 + row;
+            float4 kv4 = make_float4(0.f, 0.f, 0.f, 0.f), vv4 = kv4;
+            if (kp <= last_pos) {
+                kv4 = *reinterpret_cast<const float4*>(p.kv.pool + kv_offset(p.kv, p.layer, b, 0, h, kp) + col * 4);
+                vv4 = *reinterpret_cast<const float4*>(p.kv.pool + kv_offset(p.kv, p.layer, b, 1, h, kp) + col * 4);
+            }
+            *reinterpret_cast<float4*>(&Ks[row * LD + col * 4]) = kv4;
+            *reinterpret_cast<float4*>(&Vs[row * LD + col * 4]) = vv4;
+        }
+        __syncthreads();
+        // scores of this thread's 16 keys of the tile
+        float sc[16];
+        float mb = -INFINITY;
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) {
+            const int j = jj * 4 + c;
+            const float* kr = &Ks[j * LD];
+            float s = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) s += dot4(q4[i], *reinterpret_cast<const float4*>(kr + i * 4));
+            sc[jj] = (k0 + j <= my_pos) ? s : -INFINITY;  // causal: keys up to the query's own position
+            mb = fmaxf(mb, sc[jj]);
+        }
+        const float mn = fmaxf(m, mb);
+        if (mn > -INFINITY) {
+            const float f = expf(m - mn);
+            l *= f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                o4[i].x *= f;
+                o4[i].y *= f;
+                o4[i].z *= f;
+                o4[i].w *= f;
+            }
+#pragma unroll
+            for (int jj = 0; jj < 16; jj++) {
+                const float e = expf(sc[jj] - mn);
+                l += e;
+                const float* vr = &Vs[(jj * 4 + c) * LD];
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const float4 v = *reinterpret_cast<const float4*>(vr + i * 4);
+                    o4[i].x += e * v.x;
+                    o4[i].y += e * v.y;
+                    o4[i].z += e * v.z;
+                    o4[i].w += e * v.w;
+                }
+            }
+            m = mn;
+        }
+    }
+    // merge the four threads of the query (adjacent lanes)
+    float M = fmaxf(m, dpp_move<0xB1, 0xF>(m, m));
+    M = fmaxf(M, dpp_move<0x4E, 0xF>(M, M));
+    const float f = (m > -INFINITY) ? expf(m - M) : 0.0f;
+    l *= f;
+    l += dpp_move<0xB1, 0xF>(l, 0.0f);
+    l += dpp_move<0x4E, 0xF>(l, 0.0f);
+    const float inv = 1.0f / l;
+    float* orow = p.out + (static_cast<size_t>(b) * p.len + min(t, p.len - 1)) * p.d_model + h * HS;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float4 v = make_float4(o4[i].x * f, o4[i].y * f, o4[i].z * f, o4[i].w * f);
+        v.x += dpp_move<0xB1, 0xF>(v.x, 0.0f);
+        v.y += dpp_move<0xB1, 0xF>(v.y, 0.0f);
+        v.z += dpp_move<0xB1, 0xF>(v.z, 0.0f);
+        v.w += dpp_move<0xB1, 0xF>(v.w, 0.0f);
+        v.x += dpp_move<0x4E, 0xF>(v.x, 0.0f);
+        v.y += dpp_move<0x4E, 0xF>(v.y, 0.0f);
+        v.z += dpp_move<0x4E, 0xF>(v.z, 0.0f);
+        v.w += dpp_move<0x4E, 0xF>(v.w, 0.0f);
+        // thread c of the quad writes dims [16c, 16c + 16)
+        if (live && (i >> 2) == c)
+            reinterpret_cast<float4*>(orow)[i] = make_float4(v.x * inv, v.y * inv, v.z * inv, v.w * inv);
+    }
+}
+
 }  // namespace gh

@@ -33,19 +33,24 @@ struct GemvParams {
     const float* rope_cos;  // [max_len][head_size/2]
     const float* rope_sin;
     const DevState* st;
+    // Rows of one prompt pass: row m is token m % rows_per_seq of sequence
+    // m / rows_per_seq and sits at position pos_base + m % rows_per_seq.
+    // rows_per_seq == 0: one row per sequence, all at st->pos (a decode step).
+    int rows_per_seq;
+    int pos_base;
 };
 
 // One projected value of the fused QKV product goes to the q buffer or straight
 // into the cache row of the current position (inference.cpp:195-199).
-__device__ __forceinline__ void store_qkv(const GemvParams& p, int b, int row, float v, int pos) {
+__device__ __forceinline__ void store_qkv(const GemvParams& p, int m, int seq, int row, float v, int pos) {
     const int d = p.d_model;
     const int sec = row / d, c = row - sec * d;
     if (sec == 0) {
-        p.out[static_cast<size_t>(b) * p.out_stride + c] = v;
+        p.out[static_cast<size_t>(m) * p.out_stride + c] = v;
     } else {
         const int hs = p.kv.head_size;
         const int head = c / hs, j = c - head * hs;
-        p.kv.pool[kv_offset(p.kv, p.layer, b, sec - 1, head, pos) + j] = v;
+        p.kv.pool[kv_offset(p.kv, p.layer, seq, sec - 1, head, pos) + j] = v;
     }
 }
 
@@ -69,7 +74,13 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, int b, int ro
         // rows (2p, 2p+1) = (gate_p, up_p): hidden_p = up * silu(gate) (inference.cpp:234-239)
         p.out[static_cast<size_t>(b) * p.out_stride + (row >> 1)] = v1 * silu(v0);
     } else if constexpr (EPI == EPI_QKV) {
-        const int pos = p.st->pos;
+        int pos, seq = b;
+        if (p.rows_per_seq > 0) {
+            seq = b / p.rows_per_seq;
+            pos = p.pos_base + (b - seq * p.rows_per_seq);
+        } else {
+            pos = p.st->pos;
+        }
         float a = v0 + p.bias[row];
         float c = has1 ? v1 + p.bias[row + 1] : 0.0f;
         if (p.rope && row < 2 * p.d_model) {
@@ -83,8 +94,8 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, int b, int ro
             a = ra;
             c = rc;
         }
-        store_qkv(p, b, row, a, pos);
-        if (has1) store_qkv(p, b, row + 1, c, pos);
+        store_qkv(p, b, seq, row, a, pos);
+        if (has1) store_qkv(p, b, seq, row + 1, c, pos);
     }
 }
 
@@ -214,6 +225,28 @@ __global__ void embed_kernel(const float* __restrict__ E, const float* __restric
     float v = E[static_cast<size_t>(tok[b]) * d + j];
     if (P) v += P[static_cast<size_t>(st->pos) * d + j];
     x[static_cast<size_t>(b) * d + j] = v;
+}
+
+// The same for every token of a prompt pass: row m = seq * len + t holds token
+// t of sequence seq, at position pos_base + t.
+__global__ void embed_rows_kernel(const float* __restrict__ E, const float* __restrict__ P,
+                                  const int* __restrict__ hist, int hist_stride, int hist_base, int len,
+                                  int pos_base, float* x, int d) {
+    const int m = blockIdx.y;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= d) return;
+    const int seq = m / len, t = m - seq * len;
+    const int tok = hist[static_cast<size_t>(seq) * hist_stride + hist_base + t];
+    float v = E[static_cast<size_t>(tok) * d + j];
+    if (P) v += P[static_cast<size_t>(pos_base + t) * d + j];
+    x[static_cast<size_t>(m) * d + j] = v;
+}
+
+// rows[b] = x[b * len + len - 1]: the last position of every sequence.
+__global__ void take_last_rows_kernel(const float* __restrict__ x, int len, float* rows, int d) {
+    const int b = blockIdx.y;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < d) rows[static_cast<size_t>(b) * d + j] = x[(static_cast<size_t>(b) * len + len - 1) * d + j];
 }
 
 // pos_++ at the end of a step (inference.cpp:256).

@@ -19,6 +19,7 @@ LIB_PATH = os.path.join(PKG, "lib", "libgradhip.so")
 GH_OK, GH_ERR_RUNTIME, GH_ERR_OUT_OF_RANGE, GH_ERR_INVALID_ARGUMENT, GH_ERR_DEVICE = range(5)
 ENGINE_AUTO, ENGINE_GRAPH, ENGINE_EAGER, ENGINE_PERSISTENT = range(4)
 FLAG_PICK_GLOBAL_SCRATCH = 1
+FLAG_STEPWISE_PROMPT = 2
 
 
 class DeviceError(RuntimeError):

@@ -107,6 +107,10 @@ typedef struct gh_session_opts {
  * LDS (the path vocabularies above ~16k entries take); for testing that path. */
 enum { GH_FLAG_PICK_GLOBAL_SCRATCH = 1 };
 
+/* Feed prompts token by token (one step() each, as text_gen.cpp:44-46 does)
+ * instead of pushing all prompt tokens through each layer at once. */
+enum { GH_FLAG_STEPWISE_PROMPT = 2 };
+
 /* InferenceSession::InferenceSession (inference.cpp:121-148): allocates the
  * paged KV cache (2 * layers * max_len * d_model floats per sequence) and the
  * per-step scratch, and records the step graph. */
@@ -130,7 +134,9 @@ gh_status gh_session_logits(gh_session* s, const float** logits);
 
 /* Feeds `len` tokens per sequence (ids is batch x len, row-major) in one call;
  * equivalent to `len` step() calls (text_gen.cpp:44-46) whose logits are
- * dropped except the last.  last_logits_host may be NULL. */
+ * dropped except the last.  Prompts of 8 tokens and more go through each layer
+ * in one pass (matrix-core projections over all tokens, causal attention over
+ * the cache they fill).  last_logits_host may be NULL. */
 gh_status gh_session_prefill(gh_session* s, const int32_t* ids, int32_t len,
                              float* last_logits_host);
 

@@ -79,17 +79,35 @@ def test_batched_step_equals_per_sequence_oracle(tiny_models, name, batch):
             assert_logits_close(got[b], oss[b].step(toks[b, t]), TOL, f"{name} B{batch} seq {b} step {t}")
 
 
-def test_prefill_equals_steps(tiny_models):
-    cfg, W, om, gm = tiny_models["hs64-modern"]
-    toks = synth.uniform_tokens(3 * 30, cfg.vocab, 9).reshape(3, 30)
-    a, b = G.Session(gm, batch=3), G.Session(gm, batch=3)
-    last = a.prefill(toks)
-    for t in range(30):
-        ref = b.step(toks[:, t])
+@pytest.mark.parametrize("name", ["hs64-gpt2", "hs64-modern"])
+@pytest.mark.parametrize("batch", [1, 3])
+def test_prompt_pass_equals_steps(tiny_models, name, batch):
+    """Prompts of 8+ tokens run through each layer in one pass; the cache and the
+    last logits must be what token-by-token stepping leaves (text_gen.cpp:44-46)."""
+    cfg, W, om, gm = tiny_models[name]
+    toks = synth.uniform_tokens(batch * 30, cfg.vocab, 9).reshape(batch, 30)
+    a = G.Session(gm, batch=batch, shuffle_pages=True, page_tokens=8)
+    b = G.Session(gm, batch=batch, flags=G.FLAG_STEPWISE_PROMPT)
+    last = a.prefill(toks[:, :19])       # one pass from an empty context
+    last = a.prefill(toks[:, 19:])       # and one that continues a context
+    ref = b.prefill(toks)
     assert a.position == b.position == 30
-    assert_logits_close(last, ref, 1e-6, "prefill vs steps")
-    nxt = synth.uniform_tokens(3, cfg.vocab, 10)
-    assert_logits_close(a.step(nxt), b.step(nxt), 1e-6, "step after prefill")
+    assert_logits_close(last, ref, 2e-5, "prompt pass vs steps")
+    for seq in range(batch):
+        osess = O.Session(om)
+        for t in toks[seq]:
+            oref = osess.step(t)
+        assert_logits_close(last[seq], oref, TOL, "prompt pass vs oracle")
+        for layer in range(cfg.layers):
+            for pos in (0, 18, 19, 29):
+                for kv, row in ((0, osess.k_row(layer, pos)), (1, osess.v_row(layer, pos))):
+                    assert np.abs(a.read_kv(seq, layer, kv, pos) - row).max() <= 2e-5 * max(1.0, float(np.abs(row).max()))
+    nxt = synth.uniform_tokens(batch, cfg.vocab, 10)
+    assert_logits_close(a.step(nxt), b.step(nxt), 2e-5, "step after prompt pass")
+    # short prompts take the token-by-token route
+    c = G.Session(gm, batch=batch)
+    assert_logits_close(c.prefill(toks[:, :5]), G.Session(gm, batch=batch, flags=G.FLAG_STEPWISE_PROMPT).prefill(toks[:, :5]),
+                        1e-6, "short prompt")
 
 
 def test_errors_match_the_reference(tiny_models):
