@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     float* vin = lds + D;                 // [max(D, F)] attention output / FFN hidden
     float* ascr = vin + (F > D ? F : D);  // attention scratch: q, k, v of the head + wave partials
     int* ptab = reinterpret_cast<int*>(ascr + 192 + kPersistWaves * 68);  // [pages_per_seq]
-    const int tid = threadIdx.x, wave = tid >> 6;
+    int tid = threadIdx.x, wave = tid >> 6;
     int lane = tid & 63;
     const int wg = blockIdx.x, G = gridDim.x;
     const int V = p.V, L = p.L, H = p.H;
@@ -322,7 +322,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     const bool has_qkv = wg + G * wave < NQKV;
 
     for (int s = 0; s < p.n_steps; s++) {
-        asm volatile("" : "+v"(lane), "+v"(first));  // as in the layer loop below
+        asm volatile("" : "+v"(tid));  // as in the layer loop below
+        wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        lane = tid & 63;
+        first = wg + G * wave;
         const int pos = p.pos0 + s;
         const unsigned sb = (p.epoch + 1u + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1);
         auto tag_of = [&](int layer, int ph) {
@@ -335,6 +338,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         {
             const LayerPtrs w0l = p.layers[0];
             if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, w0l, first, pos, lane, qo);
+            else qo = QkvOperands<KD, PRO>{};  // nothing to keep alive across steps
         }
 
         // ---- token and embedding (inference.cpp:159-182)
@@ -361,7 +365,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             // Keep the compiler from hoisting every lane- and item-derived address of
             // every phase out of the layer loop (they would not fit in registers and
             // would be spilled to scratch memory): re-derive them per layer.
-            asm volatile("" : "+v"(lane), "+v"(first));
+            asm volatile("" : "+v"(tid));
+            wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+            lane = tid & 63;
+            first = wg + G * wave;
 
             // ===== phase A: norm1 + QKV (+bias, RoPE) -> q / new k / new v cells and the cache
             for (int item = first; item < NQKV; ) {
@@ -643,6 +650,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             if (l + 1 < L) {
                 const LayerPtrs wn = p.layers[l + 1];
                 if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, wn, first, pos, lane, qo);
+                else qo = QkvOperands<KD, PRO>{};
                 __syncthreads();  // xs is overwritten next
                 if (!gather_cells(p.xa, D, tag_of(l, 4), xs, p)) return;
             }
@@ -656,19 +664,19 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             float4 wr[RL][KD];
             NormRegs<KD> nf;
             load_norm<KD, PRO>(p.gf, p.bf, lane, nf);
-            if (first < nitems) {
+            // every wavefront fetches: rows past the end are clamped here and skipped on
+            // store (a conditional fetch makes the compiler spill the rows to scratch)
 #pragma unroll
-                for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(first * RL + r, V - 1), D, lane, wr[r]);
-            }
+            for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(first * RL + r, V - 1), D, lane, wr[r]);
             __syncthreads();
             if (!gather_cells(p.xa, D, tag_of(L - 1, 4), xs, p)) return;
             stamp();
             float4 h[KD];
             load_input<KD, PRO>(xs, nf, lane, h);
-            for (int item = first; item < nitems; ) {
+            auto emit = [&](int item, const float4 (&rows)[RL][KD]) {
                 float out[RL];
 #pragma unroll
-                for (int r = 0; r < RL; r++) out[r] = dot_row<KD>(wr[r], h);
+                for (int r = 0; r < RL; r++) out[r] = dot_row<KD>(rows[r], h);
                 if (lane == 0) {
 #pragma unroll
                     for (int r = 0; r < RL; r++) {
@@ -679,11 +687,15 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                         }
                     }
                 }
-                item += stride;
-                if (item < nitems) {
+            };
+            // The first item uses the rows fetched ahead; later ones (vocabularies
+            // beyond 8 rows per wavefront of the grid) fetch their own.
+            emit(first, wr);  // rows past the end are clamped on load and skipped on store
+            for (int item = first + stride; item < nitems; item += stride) {
+                float4 wl[RL][KD];
 #pragma unroll
-                    for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(item * RL + r, V - 1), D, lane, wr[r]);
-                }
+                for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(item * RL + r, V - 1), D, lane, wl[r]);
+                emit(item, wl);
             }
             // this workgroup's rows are out: signal
             __builtin_amdgcn_s_waitcnt(0);
