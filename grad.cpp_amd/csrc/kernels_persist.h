@@ -186,6 +186,15 @@ __device__ __forceinline__ float dot_row(const float4 (&w)[KV], const float4 (&h
     return wave_sum(a);
 }
 
+// The same dot product with the input vector read from LDS as it is consumed.
+template <int KV>
+__device__ __forceinline__ float dot_row_lds(const float4 (&w)[KV], const float* x, int lane) {
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < KV; i++) a += dot4(w[i], reinterpret_cast<const float4*>(x)[i * 64 + lane]);
+    return wave_sum(a);
+}
+
 // Register-resident norm parameters of one lane: the gamma (and beta) float4s
 // that line up with its slice of the row.
 template <int KV>
@@ -557,16 +566,18 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             {
                 float4 w0[KD];
                 float bo = 0.0f;
+                // idle wavefronts get defined (zero) operands: values left undefined on
+                // one path make the register allocator spill them on the other
                 if (first < D) {
                     load_row<KD>(w.wo, first, D, lane, w0);
                     bo = w.bo[first];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KD; i++) w0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
                 if (!gather_cells(p.at, D, tag_of(l, 1), vin, p)) return;
                 for (int row = first; row < D; ) {
-                    float4 h[KD];
-#pragma unroll
-                    for (int i = 0; i < KD; i++) h[i] = reinterpret_cast<const float4*>(vin)[i * 64 + lane];
-                    const float a = dot_row<KD>(w0, h);
+                    const float a = dot_row_lds<KD>(w0, vin, lane);
                     if (lane == 0) cell_put(p.xb + row, (xs[row] + bo) + a, tag_of(l, 2));
                     row += stride;
                     if (row < D) {
@@ -590,6 +601,14 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                     if (!MODERN) {
                         b0 = w.b1[2 * first];
                         b1 = w.b1[2 * first + 1];
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KD; i++) {
+                        w0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                        w1[i] = w0[i];
+                        n2.g[i] = w0[i];
+                        n2.b[i] = w0[i];
                     }
                 }
                 __syncthreads();  // every wave is done reading xs (phase C)
@@ -628,13 +647,13 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 if (first < D) {
                     load_row<KF>(w.w2, first, F, lane, w0);
                     if (!MODERN) b2 = w.b2[first];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KF; i++) w0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
                 if (!gather_cells(p.hid, F, tag_of(l, 3), vin, p)) return;
                 for (int row = first; row < D; ) {
-                    float4 h[KF];
-#pragma unroll
-                    for (int i = 0; i < KF; i++) h[i] = reinterpret_cast<const float4*>(vin)[i * 64 + lane];
-                    const float a = dot_row<KF>(w0, h);
+                    const float a = dot_row_lds<KF>(w0, vin, lane);
                     if (lane == 0) cell_put(p.xa + row, (xs[row] + b2) + a, tag_of(l, 4));
                     row += stride;
                     if (row < D) {
