@@ -620,6 +620,186 @@ __device__ inline int pick_small_wave(const float* val, const int* cidx, int S, 
     return chosen;
 }
 
+// ---------------------------------------------------------------------------
+// Fast sampler for a small top-k (the usual 20..64): no pass over radix digits
+// and no serial loop over LDS.
+//
+// Wave-level helpers: a value per lane, lane order = list order.
+
+// Lane L gets x[0] + x[1] + ... + x[L], added strictly left to right (the order
+// a serial loop over the list uses), n = list length rounded up by the caller.
+__device__ __forceinline__ float wave_prefix_in_order(float x, int n, int lane) {
+    float acc = 0.0f;
+#pragma unroll 8
+    for (int j = 0; j < n; j++) {
+        const float xj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), j));
+        acc += (lane >= j) ? xj : 0.0f;  // adding an exact zero leaves later lanes' sums untouched
+    }
+    return acc;
+}
+
+// x[0] + ... + x[n-1] left to right, in every lane.
+__device__ __forceinline__ float wave_total_in_order(float x, int n) {
+    float acc = 0.0f;
+#pragma unroll 8
+    for (int j = 0; j < n; j++) acc += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), j));
+    return acc;
+}
+
+// The sampler's tail (text_gen.cpp:156-208) for S <= 64 survivors held one per
+// lane of wavefront 0 in any order: (idx, v) with v the scaled logit.  Lanes
+// >= S pass idx = INT_MAX, v = -inf.  perm: 128 ints of LDS.  Sums are formed
+// in the reference's order: index order for the softmax denominator, the
+// renormalisation and the final walk; descending probability for top-p.
+__device__ inline int sample_survivors_wave(int idx, float v, int S, float top_p, float u, int V, int* perm) {
+    const int lane = threadIdx.x & 63;
+    const int n = min(64, (S + 7) & ~7);
+    // into index order
+    int rank = 0;
+#pragma unroll 8
+    for (int j = 0; j < n; j++) rank += (__builtin_amdgcn_readlane(idx, j) < idx);
+    perm[lane] = 0x7FFFFFFF;
+    perm[64 + lane] = __float_as_int(-INFINITY);
+    __builtin_amdgcn_wave_barrier();
+    if (lane < S) {
+        perm[rank] = idx;
+        perm[64 + rank] = __float_as_int(v);
+    }
+    __builtin_amdgcn_wave_barrier();
+    idx = perm[lane];
+    v = __int_as_float(perm[64 + lane]);
+    __builtin_amdgcn_wave_barrier();
+    const float m = wave_max(v);
+    const float e = lane < S ? expf(v - m) : 0.0f;
+    const float sum = wave_total_in_order(e, n);
+    float pr = e * (1.0f / sum);
+    if (top_p < 1.0f) {
+        // descending order of probability (ties: earlier index first)
+        int r = 0;
+#pragma unroll 8
+        for (int j = 0; j < n; j++) {
+            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pr), j));
+            r += (pj > pr) || (pj == pr && j < lane);
+        }
+        perm[lane] = 0;
+        __builtin_amdgcn_wave_barrier();
+        if (lane < n) perm[r] = __float_as_int(pr);  // r is a permutation of 0..n-1
+        __builtin_amdgcn_wave_barrier();
+        const float sorted = __int_as_float(perm[lane]);
+        __builtin_amdgcn_wave_barrier();
+        const float cum = wave_prefix_in_order(sorted, n, lane);
+        const unsigned long long reached = __ballot(lane < S && cum >= top_p);
+        // never reached: only the maximum survives
+        const int at = reached ? __ffsll(static_cast<long long>(reached)) - 1 : 0;
+        const float cutoff = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sorted), at));
+        if (!(lane < S && pr > 0.0f && pr >= cutoff)) pr = 0.0f;
+        const float total = wave_total_in_order(pr, n);
+        if (total > 0.0f) pr = pr / total;
+    }
+    if (u <= 0.0f) return 0;
+    const float cdf = wave_prefix_in_order(pr, n, lane);
+    const unsigned long long hit = __ballot(lane < S && u <= cdf);
+    if (!hit) return V - 1;
+    return __builtin_amdgcn_readlane(idx, __ffsll(static_cast<long long>(hit)) - 1);
+}
+
+constexpr int kFastCandCap = 512;
+constexpr int kFastLdsFloats = 2 * kFastCandCap + 128 + 128;  // candidates, survivors, permutation area
+
+// Temperature, top-k, softmax, top-p and the draw for 0 < top_k <= 64 over
+// val[0..V) (penalised, unscaled logits in LDS), by the whole workgroup.
+// Returns the chosen id, or -1 when this path does not apply (too many values
+// tie near the threshold); val is left untouched either way.
+//
+// The k-th largest is found without sorting: take each thread's maximum, then
+// in every wavefront the R-th largest of those (R = ceil(k / wavefronts)); the
+// smallest of these, T, has at least k values at or above it, and only a few
+// more.  Those candidates are ranked against each other.
+__device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int k, float top_p, float u,
+                                       float* work, float* red, unsigned* bcast, int* ishare) {
+    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+    float* cand_v = work;
+    int* cand_i = reinterpret_cast<int*>(work + kFastCandCap);
+    int* surv = reinterpret_cast<int*>(work + 2 * kFastCandCap);  // [64] idx, [64] value bits
+    int* perm = surv + 128;
+    float mx = -INFINITY;
+    for (int i = tid; i < V; i += nt) mx = fmaxf(mx, val[i] * inv_t);
+    const int R = (k + nw - 1) / nw;
+    float sel = mx, rest = mx;
+    for (int r = 0; r < R; r++) {
+        sel = wave_max(rest);
+        const unsigned long long at = __ballot(rest == sel);
+        if (lane == __ffsll(static_cast<long long>(at)) - 1) rest = -INFINITY;
+    }
+    if (lane == 0) red[wave] = sel;
+    if (tid == 0) {
+        ishare[1] = 0;
+        ishare[0] = 0;
+    }
+    __syncthreads();
+    float T = red[0];
+    for (int w = 1; w < nw; w++) T = fminf(T, red[w]);
+    // candidates: values >= T with their indices (slot order is arbitrary)
+    for (int i0 = 0; i0 < V; i0 += nt) {
+        const int i = i0 + tid;
+        const float x = i < V ? val[i] * inv_t : -INFINITY;
+        const bool in = i < V && x >= T;
+        const unsigned long long who = __ballot(in);
+        if (who) {
+            int base = 0;
+            if (lane == 0) base = atomicAdd(&ishare[1], __popcll(who));
+            base = __builtin_amdgcn_readfirstlane(base);
+            const int slot = base + __popcll(who & ((1ull << lane) - 1ull));
+            if (in && slot < kFastCandCap) {
+                cand_v[slot] = x;
+                cand_i[slot] = i;
+            }
+        }
+    }
+    __syncthreads();
+    const int c = ishare[1];
+    if (c > kFastCandCap || c < k) return -1;  // uniform: every thread reads the same count
+    // exact k-th largest among the candidates
+    {
+        const float mine = tid < c ? cand_v[tid] : -INFINITY;
+        int rank = 0;
+#pragma unroll 8
+        for (int j = 0; j < c; j++) {
+            const float o = cand_v[j];
+            rank += (o > mine) || (o == mine && j < tid);
+        }
+        if (tid < c && rank == k - 1) bcast[0] = __float_as_uint(mine);
+    }
+    __syncthreads();
+    const float thr = __uint_as_float(bcast[0]);
+    // survivors of the cut, ties at the threshold included (text_gen.cpp:150-154)
+    if (tid < ((c + 63) & ~63)) {
+        const bool in = tid < c && cand_v[tid] >= thr;
+        const unsigned long long who = __ballot(in);
+        if (who) {
+            int base = 0;
+            if (lane == 0) base = atomicAdd(&ishare[0], __popcll(who));
+            base = __builtin_amdgcn_readfirstlane(base);
+            const int slot = base + __popcll(who & ((1ull << lane) - 1ull));
+            if (in && slot < 64) {
+                surv[slot] = cand_i[tid];
+                surv[64 + slot] = __float_as_int(cand_v[tid]);
+            }
+        }
+    }
+    __syncthreads();
+    const int S = ishare[0];
+    if (S > 64) return -1;
+    if (tid < 64) {
+        const int idx = lane < S ? surv[lane] : 0x7FFFFFFF;
+        const float v = lane < S ? __int_as_float(surv[64 + lane]) : -INFINITY;
+        const int chosen = sample_survivors_wave(idx, v, S, top_p, u, V, perm);
+        if (tid == 0) ishare[1] = chosen;
+    }
+    __syncthreads();
+    return ishare[1];
+}
+
 constexpr int kOrderedWalkLimit = 2048;  // survivors sorted by index and walked by one lane
 
 // The pick for sequence b with the row held in `lds` ([V] values then p.sort_cap
@@ -720,8 +900,6 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
     } else {
         // ---- sample_from_logits (text_gen.cpp:135-209)
         const float inv_t = 1.0f / p.temperature;
-        for (int i = tid; i < V; i += nt) val[i] = val[i] * inv_t;
-        __syncthreads();
         float u;
         if (p.uniforms) {
             u = p.uniforms[static_cast<size_t>(b) * p.u_stride + p.pick_idx];
@@ -731,6 +909,13 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
                                              p.seed_hi ^ static_cast<unsigned>(b));
             u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
         }
+        if (p.top_k > 0 && p.top_k <= 64 && p.top_k < V && p.sort_cap >= kFastLdsFloats) {
+            const int c = sample_topk_fast(val, V, inv_t, p.top_k, p.top_p, u, srt, red, bcast, ishare);
+            __syncthreads();
+            if (c >= 0) return c;
+        }
+        for (int i = tid; i < V; i += nt) val[i] = val[i] * inv_t;
+        __syncthreads();
         if (p.dbg && threadIdx.x == 0) p.dbg[2] = __builtin_amdgcn_s_memrealtime();
         if (p.top_k > 0 && p.top_k < V) {
             const float thr = kth_largest_block(val, V, p.top_k, srt, p.sort_cap, hist256, bcast, ishare);
