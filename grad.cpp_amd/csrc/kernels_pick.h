@@ -646,84 +646,54 @@ __device__ __forceinline__ float wave_total_in_order(float x, int n) {
     return acc;
 }
 
-// The sampler's tail (text_gen.cpp:156-208) for S <= 64 survivors held one per
-// lane of wavefront 0 in any order: (idx, v) with v the scaled logit.  Lanes
-// >= S pass idx = INT_MAX, v = -inf.  perm: 128 ints of LDS.  Sums are formed
-// in the reference's order: index order for the softmax denominator, the
-// renormalisation and the final walk; descending probability for top-p.
-__device__ inline int sample_survivors_wave(int idx, float v, int S, float top_p, float u, int V, int* perm) {
-    const int lane = threadIdx.x & 63;
-    const int n = min(64, (S + 7) & ~7);
-    // into index order
-    int rank = 0;
-#pragma unroll 8
-    for (int j = 0; j < n; j++) rank += (__builtin_amdgcn_readlane(idx, j) < idx);
-    perm[lane] = 0x7FFFFFFF;
-    perm[64 + lane] = __float_as_int(-INFINITY);
-    __builtin_amdgcn_wave_barrier();
-    if (lane < S) {
-        perm[rank] = idx;
-        perm[64 + rank] = __float_as_int(v);
-    }
-    __builtin_amdgcn_wave_barrier();
-    idx = perm[lane];
-    v = __int_as_float(perm[64 + lane]);
-    __builtin_amdgcn_wave_barrier();
-    const float m = wave_max(v);
-    const float e = lane < S ? expf(v - m) : 0.0f;
-    const float sum = wave_total_in_order(e, n);
-    float pr = e * (1.0f / sum);
-    if (top_p < 1.0f) {
-        // descending order of probability (ties: earlier index first)
-        int r = 0;
-#pragma unroll 8
-        for (int j = 0; j < n; j++) {
-            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pr), j));
-            r += (pj > pr) || (pj == pr && j < lane);
-        }
-        perm[lane] = 0;
-        __builtin_amdgcn_wave_barrier();
-        if (lane < n) perm[r] = __float_as_int(pr);  // r is a permutation of 0..n-1
-        __builtin_amdgcn_wave_barrier();
-        const float sorted = __int_as_float(perm[lane]);
-        __builtin_amdgcn_wave_barrier();
-        const float cum = wave_prefix_in_order(sorted, n, lane);
-        const unsigned long long reached = __ballot(lane < S && cum >= top_p);
-        // never reached: only the maximum survives
-        const int at = reached ? __ffsll(static_cast<long long>(reached)) - 1 : 0;
-        const float cutoff = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sorted), at));
-        if (!(lane < S && pr > 0.0f && pr >= cutoff)) pr = 0.0f;
-        const float total = wave_total_in_order(pr, n);
-        if (total > 0.0f) pr = pr / total;
-    }
-    if (u <= 0.0f) return 0;
-    const float cdf = wave_prefix_in_order(pr, n, lane);
-    const unsigned long long hit = __ballot(lane < S && u <= cdf);
-    if (!hit) return V - 1;
-    return __builtin_amdgcn_readlane(idx, __ffsll(static_cast<long long>(hit)) - 1);
+constexpr int kFastCandCap = 512;
+// LDS floats the fast sampler needs: candidate values, indices and ranks, the
+// survivors (value, index, index rank) and a permutation area.
+constexpr int kFastLdsFloats = 3 * kFastCandCap + 3 * 64 + 128;
+
+// This thread's elements of val[0..V) for rounds r0 .. r0+7 (element r * nt + tid),
+// scaled, with -inf past the end; the eight LDS reads are issued together.
+__device__ __forceinline__ void load_round8(const float* val, int V, float inv_t, int r0, float (&x)[8]) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+#pragma unroll
+    for (int q = 0; q < 8; q++) x[q] = val[min((r0 + q) * nt + tid, V - 1)];
+#pragma unroll
+    for (int q = 0; q < 8; q++) x[q] = ((r0 + q) * nt + tid < V) ? x[q] * inv_t : -INFINITY;
 }
 
-constexpr int kFastCandCap = 512;
-constexpr int kFastLdsFloats = 2 * kFastCandCap + 128 + 128;  // candidates, survivors, permutation area
-
-// Temperature, top-k, softmax, top-p and the draw for 0 < top_k <= 64 over
-// val[0..V) (penalised, unscaled logits in LDS), by the whole workgroup.
-// Returns the chosen id, or -1 when this path does not apply (too many values
-// tie near the threshold); val is left untouched either way.
+// Temperature, top-k, softmax, top-p and the draw (text_gen.cpp:135-209) for
+// 0 < top_k <= 64 over val[0..V) (penalised, unscaled logits in LDS), by the
+// whole workgroup.  Returns the chosen id, or -1 when this path does not apply
+// (too many values tie near the threshold); val is left untouched either way.
 //
-// The k-th largest is found without sorting: take each thread's maximum, then
-// in every wavefront the R-th largest of those (R = ceil(k / wavefronts)); the
-// smallest of these, T, has at least k values at or above it, and only a few
-// more.  Those candidates are ranked against each other.
+// The k-th largest is found without sorting the row: take each thread's
+// maximum, then in every wavefront the R-th largest of those (R = ceil(k /
+// wavefronts)); the smallest of these, T, has at least k values at or above it
+// and only a few more.  Those candidates are ranked against each other by all
+// threads at once, which also leaves the survivors of the cut in descending
+// order.  One wavefront finishes: every sum the reference forms in index order
+// (softmax denominator, renormalisation, the final walk) or in descending order
+// (top-p) is formed in that order, lane by lane.
 __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int k, float top_p, float u,
-                                       float* work, float* red, unsigned* bcast, int* ishare) {
+                                       float* work, float* red, int* ishare) {
     const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+    const int rounds = (V + nt - 1) / nt;
+    if (rounds > 64 || nt < kFastCandCap) return -1;
     float* cand_v = work;
     int* cand_i = reinterpret_cast<int*>(work + kFastCandCap);
-    int* surv = reinterpret_cast<int*>(work + 2 * kFastCandCap);  // [64] idx, [64] value bits
-    int* perm = surv + 128;
+    int* rank = cand_i + kFastCandCap;
+    float* sv = work + 3 * kFastCandCap;  // [64] survivors, descending
+    int* si = reinterpret_cast<int*>(sv + 64);
+    int* ridx = si + 64;                  // [64] position of each survivor in index order
+    int* perm = ridx + 64;                // [128]
+
     float mx = -INFINITY;
-    for (int i = tid; i < V; i += nt) mx = fmaxf(mx, val[i] * inv_t);
+    for (int r0 = 0; r0 < rounds; r0 += 8) {
+        float x[8];
+        load_round8(val, V, inv_t, r0, x);
+#pragma unroll
+        for (int q = 0; q < 8; q++) mx = fmaxf(mx, x[q]);
+    }
     const int R = (k + nw - 1) / nw;
     float sel = mx, rest = mx;
     for (int r = 0; r < R; r++) {
@@ -732,68 +702,124 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         if (lane == __ffsll(static_cast<long long>(at)) - 1) rest = -INFINITY;
     }
     if (lane == 0) red[wave] = sel;
-    if (tid == 0) {
-        ishare[1] = 0;
-        ishare[0] = 0;
+    if (tid == 0) ishare[1] = 0;
+    if (tid < kFastCandCap) rank[tid] = 0;
+    if (tid < 64) {
+        sv[tid] = -INFINITY;
+        ridx[tid] = 0;
     }
     __syncthreads();
     float T = red[0];
     for (int w = 1; w < nw; w++) T = fminf(T, red[w]);
-    // candidates: values >= T with their indices (slot order is arbitrary)
-    for (int i0 = 0; i0 < V; i0 += nt) {
-        const int i = i0 + tid;
-        const float x = i < V ? val[i] * inv_t : -INFINITY;
-        const bool in = i < V && x >= T;
-        const unsigned long long who = __ballot(in);
-        if (who) {
-            int base = 0;
-            if (lane == 0) base = atomicAdd(&ishare[1], __popcll(who));
-            base = __builtin_amdgcn_readfirstlane(base);
-            const int slot = base + __popcll(who & ((1ull << lane) - 1ull));
-            if (in && slot < kFastCandCap) {
-                cand_v[slot] = x;
+
+    // candidates: values >= T with their indices, in arbitrary slots
+    unsigned long long mine = 0ull;
+    for (int r0 = 0; r0 < rounds; r0 += 8) {
+        float x[8];
+        load_round8(val, V, inv_t, r0, x);
+#pragma unroll
+        for (int q = 0; q < 8; q++) mine |= static_cast<unsigned long long>(x[q] >= T) << (r0 + q);
+    }
+    if (mine) {
+        int slot = atomicAdd(&ishare[1], __popcll(mine));
+        while (mine) {
+            const int r = __ffsll(static_cast<long long>(mine)) - 1;
+            mine &= mine - 1ull;
+            if (slot < kFastCandCap) {
+                const int i = r * nt + tid;
+                cand_v[slot] = val[i] * inv_t;
                 cand_i[slot] = i;
             }
+            slot++;
         }
     }
     __syncthreads();
     const int c = ishare[1];
     if (c > kFastCandCap || c < k) return -1;  // uniform: every thread reads the same count
-    // exact k-th largest among the candidates
+
+    // descending rank of every candidate (ties: lower slot first), all threads:
+    // candidate L = tid % P is compared with one slice of the list per group of P threads
     {
-        const float mine = tid < c ? cand_v[tid] : -INFINITY;
-        int rank = 0;
-#pragma unroll 8
-        for (int j = 0; j < c; j++) {
-            const float o = cand_v[j];
-            rank += (o > mine) || (o == mine && j < tid);
+        int P = 64;
+        while (P < c) P <<= 1;
+        const int parts = nt / P, L = tid & (P - 1), part = tid / P;
+        const int chunk = (c + parts - 1) / parts;
+        const int j0 = part * chunk, j1 = min(c, j0 + chunk);
+        const float me = L < c ? cand_v[L] : INFINITY;
+        int partial = 0;
+#pragma unroll 4
+        for (int j = j0; j < j1; j++) {
+            const float o = cand_v[j];  // same address in every lane: one broadcast read
+            partial += (o > me) || (o == me && j < L);
         }
-        if (tid < c && rank == k - 1) bcast[0] = __float_as_uint(mine);
+        if (L < c && partial) atomicAdd(&rank[L], partial);
     }
     __syncthreads();
-    const float thr = __uint_as_float(bcast[0]);
-    // survivors of the cut, ties at the threshold included (text_gen.cpp:150-154)
-    if (tid < ((c + 63) & ~63)) {
-        const bool in = tid < c && cand_v[tid] >= thr;
-        const unsigned long long who = __ballot(in);
-        if (who) {
-            int base = 0;
-            if (lane == 0) base = atomicAdd(&ishare[0], __popcll(who));
-            base = __builtin_amdgcn_readfirstlane(base);
-            const int slot = base + __popcll(who & ((1ull << lane) - 1ull));
-            if (in && slot < 64) {
-                surv[slot] = cand_i[tid];
-                surv[64 + slot] = __float_as_int(cand_v[tid]);
-            }
+    if (tid < c) {
+        const int r = rank[tid];
+        if (r < 64) {
+            sv[r] = cand_v[tid];
+            si[r] = cand_i[tid];
         }
     }
     __syncthreads();
-    const int S = ishare[0];
-    if (S > 64) return -1;
+    // the cut keeps ties at the threshold (text_gen.cpp:150-154)
+    const float thr = sv[k - 1];
+    const unsigned long long kept = __ballot(sv[lane] >= thr);
+    const int S = __popcll(kept);
+    if (S == 64 && c > 64) return -1;  // the ties may run past what one wavefront holds
+    {
+        // position of every survivor in index order
+        const int chunk = (S + nw - 1) / nw;
+        const int j0 = wave * chunk, j1 = min(S, j0 + chunk);
+        const int me = lane < S ? si[lane] : 0;
+        int partial = 0;
+        for (int j = j0; j < j1; j++) partial += si[j] < me;
+        if (lane < S && partial) atomicAdd(&ridx[lane], partial);
+    }
+    __syncthreads();
     if (tid < 64) {
-        const int idx = lane < S ? surv[lane] : 0x7FFFFFFF;
-        const float v = lane < S ? __int_as_float(surv[64 + lane]) : -INFINITY;
-        const int chosen = sample_survivors_wave(idx, v, S, top_p, u, V, perm);
+        const int n = min(64, (S + 7) & ~7);
+        const bool live = lane < S;
+        const float v = sv[lane];
+        const int ri = live ? ridx[lane] : lane;
+        const float e = live ? expf(v - sv[0]) : 0.0f;
+        // index-order copies of e and of the token ids
+        perm[lane] = 0;
+        perm[64 + lane] = 0x7FFFFFFF;
+        __builtin_amdgcn_wave_barrier();
+        if (live) {
+            perm[ri] = __float_as_int(e);
+            perm[64 + ri] = si[lane];
+        }
+        __builtin_amdgcn_wave_barrier();
+        const float eo = __int_as_float(perm[lane]);
+        const int io = perm[64 + lane];
+        __builtin_amdgcn_wave_barrier();
+        const float inv_sum = 1.0f / wave_total_in_order(eo, n);
+        float po = eo * inv_sum;  // index order
+        if (top_p < 1.0f) {
+            float pr = e * inv_sum;  // descending order
+            const float cum = wave_prefix_in_order(pr, n, lane);
+            const unsigned long long reached = __ballot(live && cum >= top_p);
+            // never reached: only the maximum survives
+            const int at = reached ? __ffsll(static_cast<long long>(reached)) - 1 : 0;
+            const float cutoff = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pr), at));
+            if (!(live && pr > 0.0f && pr >= cutoff)) pr = 0.0f;
+            perm[lane] = 0;
+            __builtin_amdgcn_wave_barrier();
+            if (live) perm[ri] = __float_as_int(pr);
+            __builtin_amdgcn_wave_barrier();
+            po = __int_as_float(perm[lane]);
+            const float total = wave_total_in_order(po, n);
+            if (total > 0.0f) po = po / total;
+        }
+        int chosen = 0;
+        if (u > 0.0f) {
+            const float cdf = wave_prefix_in_order(po, n, lane);
+            const unsigned long long hit = __ballot(lane < S && u <= cdf);
+            chosen = hit ? __builtin_amdgcn_readlane(io, __ffsll(static_cast<long long>(hit)) - 1) : V - 1;
+        }
         if (tid == 0) ishare[1] = chosen;
     }
     __syncthreads();
@@ -823,23 +849,38 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
     const int* hist = p.hist + static_cast<size_t>(b) * p.hist_stride;
 
     // ---- logits_with_penalty (text_gen.cpp:14-33)
+    // The window's tokens are requested first so that their latency hides behind the row's.
+    const int window = min(kPenaltyWindow, p.n_hist);
+    int window_token = -1;
+    if (tid < window) {
+        const int* hp = &hist[p.n_hist - window + tid];
+        window_token = coherent ? __hip_atomic_load(hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *hp;
+    }
     if (coherent) {
         const __amdgpu_buffer_rsrc_t rs = make_buffer(logits, static_cast<unsigned>(V) * 4u);
-        for (int i = 4 * tid; i < V; i += 4 * nt) {
-            const v4i w = coherent_load16(rs, static_cast<unsigned>(i) * 4u);
-            val[i] = __int_as_float(w.x);
-            if (i + 1 < V) val[i + 1] = __int_as_float(w.y);
-            if (i + 2 < V) val[i + 2] = __int_as_float(w.z);
-            if (i + 3 < V) val[i + 3] = __int_as_float(w.w);
+        // eight 16-byte loads per thread in flight; reads past the end return zero
+        for (int base = 4 * tid; base < V; base += 32 * nt) {
+            v4i w[8];
+#pragma unroll
+            for (int q = 0; q < 8; q++) w[q] = coherent_load16(rs, static_cast<unsigned>(base + q * 4 * nt) * 4u);
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const int i = base + q * 4 * nt;
+                if (i + 3 < V) {
+                    *reinterpret_cast<float4*>(val + i) =
+                        make_float4(__int_as_float(w[q].x), __int_as_float(w[q].y), __int_as_float(w[q].z),
+                                    __int_as_float(w[q].w));
+                } else {
+                    if (i < V) val[i] = __int_as_float(w[q].x);
+                    if (i + 1 < V) val[i + 1] = __int_as_float(w[q].y);
+                    if (i + 2 < V) val[i + 2] = __int_as_float(w[q].z);
+                }
+            }
         }
     } else {
         for (int i = tid; i < V; i += nt) val[i] = logits[i];
     }
-    const int window = min(kPenaltyWindow, p.n_hist);
-    if (tid < window) {
-        const int* hp = &hist[p.n_hist - window + tid];
-        win_tok[tid] = coherent ? __hip_atomic_load(hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *hp;
-    }
+    if (tid < window) win_tok[tid] = window_token;
     if (p.dbg && threadIdx.x == 0) p.dbg[0] = __builtin_amdgcn_s_memrealtime();
     __syncthreads();
     if (p.penalty != 1.0f && tid < 64) {
@@ -910,7 +951,7 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
             u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
         }
         if (p.top_k > 0 && p.top_k <= 64 && p.top_k < V && p.sort_cap >= kFastLdsFloats) {
-            const int c = sample_topk_fast(val, V, inv_t, p.top_k, p.top_p, u, srt, red, bcast, ishare);
+            const int c = sample_topk_fast(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare);
             __syncthreads();
             if (c >= 0) return c;
         }
