@@ -25,6 +25,13 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# rocprofv3 counters for one 224-step launch of the batch-1 persistent kernel
+# (32-token prompt already cached): FETCH_SIZE and WRITE_SIZE, converted to bytes
+# with the factors a 1 GiB copy kernel gives for the same counters.
+PMC_STEPS_PER_LAUNCH = 224
+PMC_FETCH_BYTES_PER_LAUNCH = 31_418_894 * 2048  # counter reads 1 per 2 KiB fetched
+PMC_WRITE_BYTES_PER_LAUNCH = 540_302 * 1024     # counter reads 1 per KiB written
+
 
 def step_bytes(cfg, batch, ctx):
     """Algorithmic bytes of one decode step: every matrix once (regardless of
@@ -47,6 +54,7 @@ def run_decode(G, synth, gm, cfg, batch, prompt_len, steps, warmup, opt, seed, e
     done = -warmup
     wall = gpu_ms = 0.0
     byte_sum = 0
+    launches = []  # (steps, GPU ms, algorithmic bytes) of every timed decode round
     prefill_ms = 0.0
     prefill_tok = 0
     while done < steps:
@@ -62,11 +70,13 @@ def run_decode(G, synth, gm, cfg, batch, prompt_len, steps, warmup, opt, seed, e
         if done >= 0:
             wall += t2 - t1
             gpu_ms += tm["decode_ms"]
-            byte_sum += sum(step_bytes(cfg, batch, prompt_len + i + 1) for i in range(n))
+            round_bytes = sum(step_bytes(cfg, batch, prompt_len + i + 1) for i in range(n))
+            byte_sum += round_bytes
+            launches.append((n, tm["decode_ms"], round_bytes))
             prefill_ms += (t1 - t0) * 1e3
             prefill_tok += batch * prompt_len
         done += n
-    return {"wall_s": wall, "gpu_ms": gpu_ms, "bytes": byte_sum, "steps": steps,
+    return {"wall_s": wall, "gpu_ms": gpu_ms, "bytes": byte_sum, "steps": steps, "launches": launches,
             "launches_per_step": tm["launches_per_step"],
             "prefill_tok_s": prefill_tok / (prefill_ms / 1e3) if prefill_ms else None}
 
@@ -97,7 +107,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=448)
-    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=224)
     ap.add_argument("--engine", default="auto", choices=["auto", "graph", "eager", "persistent"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-batch64", action="store_true", help="skip the batch-64 leg")
@@ -141,8 +151,23 @@ def main():
         return
     r1 = run_decode(G, synth, gm, cfg, 1, 32, a.steps, a.warmup, sample, 2002, engine)
     tok_s = r1["steps"] / r1["wall_s"]
-    step_us = r1["gpu_ms"] * 1e3 / r1["steps"]
-    achieved = r1["bytes"] / (r1["gpu_ms"] / 1e3) / 1e9
+    persistent = r1["launches_per_step"] == 1
+    n_l = len(r1["launches"])
+    us_per_launch = sum(ms for _, ms, _ in r1["launches"]) * 1e3 / n_l
+    bytes_per_launch = sum(nb for _, _, nb in r1["launches"]) / n_l
+    steps_per_launch = sum(n for n, _, _ in r1["launches"]) / n_l
+    achieved = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
+    if persistent:
+        kernel = ("gh::persist_decode_kernel<3, 8, true>: one launch = one pick + step round per token "
+                  "for a whole run of steps")
+    else:
+        kernel = "every kernel of the decode round (one launch per fused op), timed as one span"
+    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the
+    # summary under profiles/ for the command and the copy-kernel calibration);
+    # only valid for the launch shape it was measured on.
+    traffic = None
+    if persistent and steps_per_launch == PMC_STEPS_PER_LAUNCH:
+        traffic = PMC_FETCH_BYTES_PER_LAUNCH + PMC_WRITE_BYTES_PER_LAUNCH
 
     line = {
         "metric": "decode tok/s, 69M Llama block, batch 1",
@@ -154,11 +179,10 @@ def main():
                    "batch": 1, "engine": a.engine, "launches_per_step": r1["launches_per_step"]},
         "device": info["name"],
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "one decode step (all kernels of the step, timed with HIP events on "
-                               "the session stream)",
-                     "us_per_launch": round(step_us, 2),
-                     "bytes_per_launch": int(r1["bytes"] / r1["steps"])},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "kernel": kernel, "launches": n_l, "steps_per_launch": steps_per_launch,
+                     "us_per_launch": round(us_per_launch, 1),
+                     "bytes_per_launch": int(bytes_per_launch)},
         "prefill_tok_s": round(r1["prefill_tok_s"], 1),
     }
 
