@@ -392,8 +392,6 @@ struct Session {
                 if (std::FILE* f = std::fopen(std::getenv("GRADHIP_PROF_DUMP"), "w")) {
                     for (size_t i = 0; i < host.size() / 2 && host[i]; i++) std::fprintf(f, "%llu\n", host[i]);
                     std::fprintf(f, "0\n");
-                    for (size_t i = host.size() - 16; i < host.size() - 8; i++) std::fprintf(f, "%llu\n", host[i]);
-                    std::fprintf(f, "0\n");
                     for (size_t i = host.size() / 2; i + 3 < host.size() && host[i]; i += 4)
                         std::fprintf(f, "%llu\n%llu\n%llu\n", host[i + 2], host[i], host[i + 1]);
                     std::fclose(f);

@@ -72,14 +72,28 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
     if (n0 >= p.N) return;
     const int K = p.K, kq = K / KW;  // this wavefront's share of K
     const int j = lane & 15, g = lane >> 4;
+    // Fetch layout: four neighbouring lanes read 64 contiguous bytes of one row
+    // (lane = 4 * row + chunk), which the memory pipeline serves far faster than
+    // the MFMA operand layout (lane = 16 * chunk + row) where neighbouring lanes
+    // sit in different rows.  to_operand() moves a fetched float4 to the lane that
+    // feeds it to the matrix core.
+    const int fr = lane >> 2, fc = lane & 3;
+    const int from_lane = (j * 4 + g) * 4;  // byte address of the source lane for ds_bpermute
+    auto to_operand = [&](const float4& v) {
+        return make_float4(
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.x))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.y))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.z))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.w))));
+    };
     const float* wp[NT];
     const float* ap[MT];
 #pragma unroll
     for (int t = 0; t < NT; t++)
-        wp[t] = p.W + static_cast<size_t>(min(n0 + t * 16 + j, p.N - 1)) * K + wave * kq + g * 4;
+        wp[t] = p.W + static_cast<size_t>(min(n0 + t * 16 + fr, p.N - 1)) * K + wave * kq + fc * 4;
 #pragma unroll
     for (int t = 0; t < MT; t++)
-        ap[t] = p.in + static_cast<size_t>(min(m0 + t * 16 + j, M - 1)) * p.in_stride + wave * kq + g * 4;
+        ap[t] = p.in + static_cast<size_t>(min(m0 + t * 16 + fr, M - 1)) * p.in_stride + wave * kq + fc * 4;
     const float* gp = RMS ? p.gamma + wave * kq + g * 4 : nullptr;
     v4f acc[MT][NT];
     float ss[MT];
@@ -92,14 +106,17 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
     // K-steps of loads in flight: as many as ~100 registers of fragments allow
     constexpr int UNROLL = (MT + NT + 1) <= 3 ? 8 : (MT + NT + 1) <= 6 ? 4 : 2;
 
-    auto consume = [&](const float4 (&a)[MT], const float4 (&b)[NT], const float4& g4) {
-        float4 as[MT];
+    auto consume = [&](const float4 (&a_in)[MT], const float4 (&b_in)[NT], const float4& g4) {
+        float4 as[MT], b[NT];
+#pragma unroll
+        for (int u = 0; u < NT; u++) b[u] = to_operand(b_in[u]);
 #pragma unroll
         for (int t = 0; t < MT; t++) {
-            as[t] = a[t];
+            const float4 a = to_operand(a_in[t]);
+            as[t] = a;
             if (RMS) {
-                ss[t] += dot4(a[t], a[t]);
-                as[t] = make_float4(a[t].x * g4.x, a[t].y * g4.y, a[t].z * g4.z, a[t].w * g4.w);
+                ss[t] += dot4(a, a);
+                as[t] = make_float4(a.x * g4.x, a.y * g4.y, a.z * g4.z, a.w * g4.w);
             }
         }
 #pragma unroll
@@ -188,21 +205,27 @@ inline void launch_gemm16_as(const GemvParams& p, int M, hipStream_t st) {
                        st, p, M, m_groups);
 }
 
-// K is split over 8 wavefronts when that leaves each a multiple of 16.
+// Tile shapes by measurement on the decode shapes (M = 64 rows): every launch
+// is bound by latency (kernel start, one trip to memory, the merge across the K
+// split), not by the weights, so small tiles on many workgroups win; long row
+// blocks (a prompt pass) take the whole 64-row tile so each weight row is
+// fetched once per workgroup.  K is split over 8 wavefronts when that leaves
+// each a multiple of 16.
 template <int EPI, bool RMS>
 inline void launch_gemm16(const GemvParams& p, int M, hipStream_t st) {
     const bool k8 = p.K % 128 == 0;
     if (p.N <= 1024 || M <= 16) {
         if (k8) launch_gemm16_as<EPI, RMS, 1, 1, 8>(p, M, st);
         else launch_gemm16_as<EPI, RMS, 1, 1, 4>(p, M, st);
-    } else if (M <= 32) {
+    } else if (p.N > 8192) {
+        if (M <= 64) launch_gemm16_as<EPI, RMS, 2, 2, 4>(p, M, st);
+        else launch_gemm16_as<EPI, RMS, 4, 2, 4>(p, M, st);
+    } else if (M <= 64) {
         if (k8) launch_gemm16_as<EPI, RMS, 2, 1, 8>(p, M, st);
         else launch_gemm16_as<EPI, RMS, 2, 1, 4>(p, M, st);
-    } else if (p.N <= 8192) {
+    } else {
         if (k8) launch_gemm16_as<EPI, RMS, 4, 1, 8>(p, M, st);
         else launch_gemm16_as<EPI, RMS, 4, 1, 4>(p, M, st);
-    } else {
-        launch_gemm16_as<EPI, RMS, 4, 2, 4>(p, M, st);
     }
 }
 

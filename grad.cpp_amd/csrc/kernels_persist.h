@@ -157,12 +157,7 @@ __device__ inline bool persist_pick(const PersistParams& p, float* lds, int i_pi
     PickParams pk = p.pick;
     pk.n_hist = p.pick.n_hist + i_pick;
     pk.pick_idx = p.pick.pick_idx + i_pick;
-    pk.dbg = (p.prof && i_pick == 100) ? p.prof + p.prof_cap - 16 : nullptr;
-#ifndef PROBE_NO_PICK
     const int chosen = pick_lds_body(pk, 0, lds, true);
-#else
-    const int chosen = 0;
-#endif
     if (tid == 0) {
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         cell_put(p.tokc, __int_as_float(chosen), tok_tag);
@@ -414,7 +409,6 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             stamp();
 
             // ===== phase B: attention of one head per workgroup (inference.cpp:211-225)
-#ifndef PROBE_NO_ATTN
             if (wg < H) {
                 const int hd = wg;
                 float* qkv = ascr;         // [3][64]: q, key and value of the current position
@@ -559,7 +553,6 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 }
                 __syncthreads();
             }
-#endif
             stamp();
 
             // ===== phase C: x += b_o + attn @ W_o
@@ -675,7 +668,6 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             }
         }
 
-#ifndef PROBE_NO_LOGITS
         if (want_logits) {
             // ===== final norm + logits = h @ E^T (inference.cpp:251-254); the rows of
             // E are fetched while the last layer's x is still being exchanged.
@@ -723,9 +715,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             if (tid == 0)
                 __hip_atomic_fetch_add(&p.ctl->arrive[(wg & 15) * 32], 1u, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
-        } else
-#endif
-        {
+        } else {
             // nobody needs this step's logits: the last x stays in its cells
             stamp();
         }

@@ -36,7 +36,6 @@ struct PickParams {
     unsigned seed_lo, seed_hi;
     int sort_cap;  // floats of LDS available for the descending sort (power of two)
     int* err;      // set to 1 when top-p needs a sort larger than sort_cap
-    unsigned long long* dbg;  // optional timestamps (developer aid)
 };
 
 __device__ __forceinline__ unsigned mulhi32(unsigned a, unsigned b) { return __umulhi(a, b); }
@@ -718,7 +717,8 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         float x[8];
         load_round8(val, V, inv_t, r0, x);
 #pragma unroll
-        for (int q = 0; q < 8; q++) mine |= static_cast<unsigned long long>(x[q] >= T) << (r0 + q);
+        for (int q = 0; q < 8; q++)
+            mine |= static_cast<unsigned long long>(x[q] >= T && (r0 + q) * nt + tid < V) << (r0 + q);
     }
     if (mine) {
         int slot = atomicAdd(&ishare[1], __popcll(mine));
@@ -881,7 +881,6 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
         for (int i = tid; i < V; i += nt) val[i] = logits[i];
     }
     if (tid < window) win_tok[tid] = window_token;
-    if (p.dbg && threadIdx.x == 0) p.dbg[0] = __builtin_amdgcn_s_memrealtime();
     __syncthreads();
     if (p.penalty != 1.0f && tid < 64) {
         // lane e holds window entry e; a token is handled by its first occurrence,
@@ -900,8 +899,6 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
         }
     }
     __syncthreads();
-
-    if (p.dbg && threadIdx.x == 0) p.dbg[1] = __builtin_amdgcn_s_memrealtime();
     int chosen;
     if (p.greedy) {
         float best = -INFINITY;
@@ -957,10 +954,8 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
         }
         for (int i = tid; i < V; i += nt) val[i] = val[i] * inv_t;
         __syncthreads();
-        if (p.dbg && threadIdx.x == 0) p.dbg[2] = __builtin_amdgcn_s_memrealtime();
         if (p.top_k > 0 && p.top_k < V) {
             const float thr = kth_largest_block(val, V, p.top_k, srt, p.sort_cap, hist256, bcast, ishare);
-            if (p.dbg && threadIdx.x == 0) p.dbg[3] = __builtin_amdgcn_s_memrealtime();
             // Survivors of the cut (ties at the threshold included).  When they fit
             // one wavefront the rest of the sampler runs there.
             int* cidx = reinterpret_cast<int*>(srt);
@@ -973,7 +968,6 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
                 }
             }
             __syncthreads();
-            if (p.dbg && threadIdx.x == 0) p.dbg[4] = __builtin_amdgcn_s_memrealtime();
             const int S0 = ishare[1];
             if (S0 <= 64 && p.sort_cap >= 512) {
                 if (tid < 64) {
@@ -981,7 +975,6 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
                     if (tid == 0) ishare[0] = c;
                 }
                 __syncthreads();
-                if (p.dbg && threadIdx.x == 0) p.dbg[5] = __builtin_amdgcn_s_memrealtime();
                 const int c = ishare[0];
                 __syncthreads();
                 return c;
