@@ -625,16 +625,19 @@ __device__ inline int pick_small_wave(const float* val, const int* cidx, int S, 
 //
 // Wave-level helpers: a value per lane, lane order = list order.
 
-// Lane L gets x[0] + x[1] + ... + x[L], added strictly left to right (the order
-// a serial loop over the list uses), n = list length rounded up by the caller.
-__device__ __forceinline__ float wave_prefix_in_order(float x, int n, int lane) {
+// Number of prefixes x[0], x[0] + x[1], ... (added strictly left to right, the
+// order a serial loop over the list uses) that are below thr.  The x are >= 0, so
+// the prefixes never decrease and this is the index of the first prefix that
+// reaches thr (n when none does).  Same value in every lane.
+__device__ __forceinline__ int wave_prefixes_below(float x, int n, float thr) {
     float acc = 0.0f;
+    int below = 0;
 #pragma unroll 8
     for (int j = 0; j < n; j++) {
-        const float xj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), j));
-        acc += (lane >= j) ? xj : 0.0f;  // adding an exact zero leaves later lanes' sums untouched
+        acc += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), j));
+        below += (acc < thr) ? 1 : 0;
     }
-    return acc;
+    return below;
 }
 
 // x[0] + ... + x[n-1] left to right, in every lane.
@@ -650,16 +653,6 @@ constexpr int kFastCandCap = 512;
 // survivors (value, index, index rank) and a permutation area.
 constexpr int kFastLdsFloats = 3 * kFastCandCap + 3 * 64 + 128;
 
-// This thread's elements of val[0..V) for rounds r0 .. r0+7 (element r * nt + tid),
-// scaled, with -inf past the end; the eight LDS reads are issued together.
-__device__ __forceinline__ void load_round8(const float* val, int V, float inv_t, int r0, float (&x)[8]) {
-    const int tid = threadIdx.x, nt = blockDim.x;
-#pragma unroll
-    for (int q = 0; q < 8; q++) x[q] = val[min((r0 + q) * nt + tid, V - 1)];
-#pragma unroll
-    for (int q = 0; q < 8; q++) x[q] = ((r0 + q) * nt + tid < V) ? x[q] * inv_t : -INFINITY;
-}
-
 // Temperature, top-k, softmax, top-p and the draw (text_gen.cpp:135-209) for
 // 0 < top_k <= 64 over val[0..V) (penalised, unscaled logits in LDS), by the
 // whole workgroup.  Returns the chosen id, or -1 when this path does not apply
@@ -673,11 +666,16 @@ __device__ __forceinline__ void load_round8(const float* val, int V, float inv_t
 // order.  One wavefront finishes: every sum the reference forms in index order
 // (softmax denominator, renormalisation, the final walk) or in descending order
 // (top-p) is formed in that order, lane by lane.
+// NT = threads of the workgroup (compile time, so that a thread's elements sit
+// at immediate offsets and stay in registers between the two passes); needs
+// V <= 32 * NT and V + NT floats of readable LDS behind val.
+template <int NT>
 __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int k, float top_p, float u,
                                        float* work, float* red, int* ishare) {
-    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
-    const int rounds = (V + nt - 1) / nt;
-    if (rounds > 64 || nt < kFastCandCap) return -1;
+    constexpr int nt = NT, nw = NT / 64, ROUNDS = 32;
+    static_assert(NT >= kFastCandCap, "every candidate needs a thread");
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (V > ROUNDS * NT) return -1;
     float* cand_v = work;
     int* cand_i = reinterpret_cast<int*>(work + kFastCandCap);
     int* rank = cand_i + kFastCandCap;
@@ -686,13 +684,20 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
     int* ridx = si + 64;                  // [64] position of each survivor in index order
     int* perm = ridx + 64;                // [128]
 
-    float mx = -INFINITY;
-    for (int r0 = 0; r0 < rounds; r0 += 8) {
-        float x[8];
-        load_round8(val, V, inv_t, r0, x);
+    // element r * NT + tid of the row, scaled; -inf past the end
+    float x[ROUNDS];
+    const float* mine_base = val + tid;
 #pragma unroll
-        for (int q = 0; q < 8; q++) mx = fmaxf(mx, x[q]);
+    for (int r = 0; r < ROUNDS; r++) {
+        x[r] = -INFINITY;
+        if (r * NT < V) {  // uniform; the last round may read (and discard) floats just past V
+            const float raw = mine_base[r * NT];
+            x[r] = (tid < V - r * NT) ? raw * inv_t : -INFINITY;
+        }
     }
+    float mx = x[0];
+#pragma unroll
+    for (int r = 1; r < ROUNDS; r++) mx = fmaxf(mx, x[r]);
     const int R = (k + nw - 1) / nw;
     float sel = mx, rest = mx;
     for (int r = 0; r < R; r++) {
@@ -711,20 +716,16 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
     float T = red[0];
     for (int w = 1; w < nw; w++) T = fminf(T, red[w]);
 
+    if (!(T > -INFINITY)) return -1;  // some wavefront has fewer than R finite values
     // candidates: values >= T with their indices, in arbitrary slots
-    unsigned long long mine = 0ull;
-    for (int r0 = 0; r0 < rounds; r0 += 8) {
-        float x[8];
-        load_round8(val, V, inv_t, r0, x);
+    unsigned mine = 0u;
 #pragma unroll
-        for (int q = 0; q < 8; q++)
-            mine |= static_cast<unsigned long long>(x[q] >= T && (r0 + q) * nt + tid < V) << (r0 + q);
-    }
+    for (int r = 0; r < ROUNDS; r++) mine |= static_cast<unsigned>(x[r] >= T) << r;
     if (mine) {
-        int slot = atomicAdd(&ishare[1], __popcll(mine));
+        int slot = atomicAdd(&ishare[1], __popc(mine));
         while (mine) {
-            const int r = __ffsll(static_cast<long long>(mine)) - 1;
-            mine &= mine - 1ull;
+            const int r = __ffs(mine) - 1;
+            mine &= mine - 1u;
             if (slot < kFastCandCap) {
                 const int i = r * nt + tid;
                 cand_v[slot] = val[i] * inv_t;
@@ -800,10 +801,10 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         float po = eo * inv_sum;  // index order
         if (top_p < 1.0f) {
             float pr = e * inv_sum;  // descending order
-            const float cum = wave_prefix_in_order(pr, n, lane);
-            const unsigned long long reached = __ballot(live && cum >= top_p);
-            // never reached: only the maximum survives
-            const int at = reached ? __ffsll(static_cast<long long>(reached)) - 1 : 0;
+            // first position whose running sum reaches top_p; never reached: only the
+            // maximum survives
+            const int reach = wave_prefixes_below(pr, n, top_p);
+            const int at = reach < S ? reach : 0;
             const float cutoff = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pr), at));
             if (!(live && pr > 0.0f && pr >= cutoff)) pr = 0.0f;
             perm[lane] = 0;
@@ -816,9 +817,8 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         }
         int chosen = 0;
         if (u > 0.0f) {
-            const float cdf = wave_prefix_in_order(po, n, lane);
-            const unsigned long long hit = __ballot(lane < S && u <= cdf);
-            chosen = hit ? __builtin_amdgcn_readlane(io, __ffsll(static_cast<long long>(hit)) - 1) : V - 1;
+            const int hit = wave_prefixes_below(po, n, u);  // first i with u <= cumulative
+            chosen = hit < S ? __builtin_amdgcn_readlane(io, hit) : V - 1;
         }
         if (tid == 0) ishare[1] = chosen;
     }
@@ -838,6 +838,7 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
     __shared__ unsigned hist256[256];
     __shared__ unsigned bcast[2];
     __shared__ int win_tok[kPenaltyWindow];
+    __shared__ int pen_before[64], pen_count[64];
     __shared__ float fshare[2];
     __shared__ int ishare[2];
 
@@ -881,24 +882,39 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
         for (int i = tid; i < V; i += nt) val[i] = logits[i];
     }
     if (tid < window) win_tok[tid] = window_token;
-    __syncthreads();
-    if (p.penalty != 1.0f && tid < 64) {
-        // lane e holds window entry e; a token is handled by its first occurrence,
-        // which applies the penalty once per occurrence
-        const int id = tid < window ? win_tok[tid] : -1 - tid;
-        int before = 0, count = 0;
-        for (int e = 0; e < kPenaltyWindow; e++) {
-            const int other = __builtin_amdgcn_readlane(id, e);
-            before += (e < tid && other == id);
-            count += (other == id);
-        }
-        if (tid < window && before == 0) {
-            float v = val[id];
-            for (int c = 0; c < count; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
-            val[id] = v;
-        }
+    if (tid < 64) {
+        pen_before[tid] = 0;
+        pen_count[tid] = 0;
     }
     __syncthreads();
+    if (p.penalty != 1.0f) {
+        // Entry e of the window is handled by its first occurrence, which applies
+        // the penalty once per occurrence.  Every wavefront compares all entries
+        // with one slice of the window.
+        const int lane = tid & 63, nw = nt >> 6, wave = tid >> 6;
+        const int slice = (window + nw - 1) / nw;
+        const int j0 = wave * slice, j1 = min(window, j0 + slice);
+        const int id = lane < window ? win_tok[lane] : -1 - lane;
+        int before = 0, count = 0;
+        for (int e = j0; e < j1; e++) {
+            const int other = win_tok[e];
+            before += (e < lane && other == id);
+            count += (other == id);
+        }
+        if (lane < window && count) {
+            if (before) atomicAdd(&pen_before[lane], before);
+            atomicAdd(&pen_count[lane], count);
+        }
+        __syncthreads();
+        if (tid < window && pen_before[tid] == 0) {
+            const int tok = win_tok[tid], count_all = pen_count[tid];
+            float v = val[tok];
+            for (int c = 0; c < count_all; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
+            val[tok] = v;
+        }
+        __syncthreads();
+    }
+
     int chosen;
     if (p.greedy) {
         float best = -INFINITY;
@@ -947,8 +963,11 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
                                              p.seed_hi ^ static_cast<unsigned>(b));
             u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
         }
-        if (p.top_k > 0 && p.top_k <= 64 && p.top_k < V && p.sort_cap >= kFastLdsFloats) {
-            const int c = sample_topk_fast(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare);
+        if (p.top_k > 0 && p.top_k <= 64 && p.top_k < V && p.sort_cap >= kFastLdsFloats && p.sort_cap >= nt
+            && (nt == 512 || nt == 1024)) {
+            const int c = nt == 512
+                              ? sample_topk_fast<512>(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare)
+                              : sample_topk_fast<1024>(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare);
             __syncthreads();
             if (c >= 0) return c;
         }
