@@ -86,12 +86,15 @@ __device__ __forceinline__ void coherent_store(float* p, float v) {
 }
 
 // Workgroup-wide: waits until cells [0, n) carry `tag`, copying the values to
-// dst (LDS).  Returns false when the wait was abandoned (the kernel must exit).
+// dst (LDS).  Every thread polls only its own cells and stops as soon as they
+// have arrived; the workgroup meets once at the end.  Returns false when the wait
+// was abandoned (the kernel must exit).
 __device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float* dst,
                                     const PersistParams& p) {
     const __amdgpu_buffer_rsrc_t rs = make_buffer(src, static_cast<unsigned>(n) * 8u);
     const int itag = static_cast<int>(tag);
     unsigned spins = 0;
+    bool failed = false;
     for (;;) {
         bool ok = true;
         // two cells per 16-byte load, all of a thread's loads in flight together
@@ -101,19 +104,23 @@ __device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float*
             dst[i] = __int_as_float(w.x);
             if (i + 1 < n) dst[i + 1] = __int_as_float(w.z);
         }
-        if (__syncthreads_and(ok)) return true;
+        if (ok) break;
         ++spins;
-        bool give_up = spins > p.spin_limit;
-        if ((spins & 63u) == 0u)
-            give_up = give_up || __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-        if (__syncthreads_or(give_up)) {
-            if (threadIdx.x == 0) {
-                __hip_atomic_store(&p.ctl->where, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            return false;
+        if (spins > p.spin_limit
+            || ((spins & 63u) == 0u
+                && __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
+            failed = true;
+            break;
         }
     }
+    if (__syncthreads_or(failed)) {
+        if (threadIdx.x == 0) {
+            __hip_atomic_store(&p.ctl->where, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return false;
+    }
+    return true;
 }
 
 // One pick by workgroup 0 (text_gen.cpp:48-61 / :80-86): waits until every
@@ -438,28 +445,31 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 {
                     const unsigned t = tag_of(l, 0);
                     unsigned spins = 0;
-                    for (;;) {
-                        bool ok = true;
-                        if (tid < 96) {
-                            const int seg = tid >> 5, j = (tid & 31) * 2;
-                            const Cell* src = (seg == 0 ? p.q : seg == 1 ? p.kn : p.vn) + hd * HS;
-                            const v4i w = coherent_load16(make_buffer(src, HS * 8u), static_cast<unsigned>(j) * 8u);
-                            ok = w.y == static_cast<int>(t) && w.w == static_cast<int>(t);
+                    bool failed = false;
+                    if (tid < 96) {
+                        const int seg = tid >> 5, j = (tid & 31) * 2;
+                        const Cell* src = (seg == 0 ? p.q : seg == 1 ? p.kn : p.vn) + hd * HS;
+                        const __amdgpu_buffer_rsrc_t rs = make_buffer(src, HS * 8u);
+                        for (;;) {
+                            const v4i w = coherent_load16(rs, static_cast<unsigned>(j) * 8u);
                             qkv[seg * 64 + j] = __int_as_float(w.x);
                             qkv[seg * 64 + j + 1] = __int_as_float(w.z);
-                        }
-                        if (__syncthreads_and(ok)) break;
-                        ++spins;
-                        bool give_up = spins > p.spin_limit;
-                        if ((spins & 63u) == 0u)
-                            give_up = give_up || __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-                        if (__syncthreads_or(give_up)) {
-                            if (tid == 0) {
-                                __hip_atomic_store(&p.ctl->where, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                                __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            if (w.y == static_cast<int>(t) && w.w == static_cast<int>(t)) break;
+                            ++spins;
+                            if (spins > p.spin_limit
+                                || ((spins & 63u) == 0u
+                                    && __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
+                                failed = true;
+                                break;
                             }
-                            return;
                         }
+                    }
+                    if (__syncthreads_or(failed)) {
+                        if (tid == 0) {
+                            __hip_atomic_store(&p.ctl->where, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                        return;
                     }
                 }
                 const float4 q4 = reinterpret_cast<const float4*>(qkv)[dl];
