@@ -130,33 +130,36 @@ __device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float*
 __device__ inline bool persist_pick(const PersistParams& p, float* lds, int i_pick,
                                     unsigned arrive_gen, unsigned tok_tag, bool wait_logits) {
     if (blockIdx.x != 0) return true;
-    __shared__ unsigned total;
     const int tid = threadIdx.x;
     if (p.prof && i_pick < 1024 && tid == 0) p.prof[p.prof_cap / 2 + 4 * i_pick + 2] = __builtin_amdgcn_s_memrealtime();
     if (wait_logits) {
-        unsigned spins = 0;
-        for (;;) {
-            unsigned v = 0;
-            if (tid < 16)
-                v = __hip_atomic_load(&p.ctl->arrive[tid * 32], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (tid < 64) {
+        // one wavefront watches the 16 arrival counters; the workgroup meets once
+        bool failed = false;
+        if (tid < 64) {
+            const unsigned target = arrive_gen * gridDim.x;
+            unsigned spins = 0;
+            for (;;) {
+                unsigned v = 0;
+                if (tid < 16)
+                    v = __hip_atomic_load(&p.ctl->arrive[tid * 32], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-                for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-            }
-            if (tid == 0) total = v;
-            __syncthreads();
-            const bool done = total >= arrive_gen * gridDim.x;
-            __syncthreads();
-            if (done) break;
-            const bool aborted = (spins & 63u) == 63u
-                                 && __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-            if (__syncthreads_or(++spins > p.spin_limit || aborted)) {
-                if (tid == 0) {
-                    __hip_atomic_store(&p.ctl->where, 0xFFFFFFFEu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+                if (__builtin_amdgcn_readfirstlane(v) >= target) break;
+                ++spins;
+                if (spins > p.spin_limit
+                    || ((spins & 63u) == 63u
+                        && __hip_atomic_load(&p.ctl->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
+                    failed = true;
+                    break;
                 }
-                return false;
             }
+        }
+        if (__syncthreads_or(failed)) {
+            if (tid == 0) {
+                __hip_atomic_store(&p.ctl->where, 0xFFFFFFFEu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            return false;
         }
     }
     unsigned long long* pp = (p.prof && i_pick < 1024) ? p.prof + p.prof_cap / 2 + 4 * i_pick : nullptr;
