@@ -912,7 +912,7 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
         if (s.engine == GH_ENGINE_PERSISTENT && why) throw ApiError{GH_ERR_INVALID_ARGUMENT, why};
         if (s.engine == GH_ENGINE_AUTO) s.engine = why ? GH_ENGINE_GRAPH : GH_ENGINE_PERSISTENT;
         if (s.engine == GH_ENGINE_PERSISTENT) {
-            const size_t work = d + std::max(d, F) + 192 + kPersistWaves * 68 + s.pages_per_seq;
+            const size_t work = d + std::max(d, F) + 192 + kPersistWaves * 4 * 68 + s.pages_per_seq;
             s.persist_lds = std::max(work, static_cast<size_t>(s.pick_lds_floats)) * sizeof(float);
             s.persist_grid = std::min(prop.multiProcessorCount, 256);
             dev_alloc(s.cells, 6 * d + F + 1);

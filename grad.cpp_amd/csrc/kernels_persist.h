@@ -17,6 +17,7 @@
 // (kernels_gemv.h, kernels_attn.h), i.e. src/transformer/inference.cpp:150-258.
 #pragma once
 
+#include "kernels_attn.h"
 #include "kernels_common.h"
 #include "kernels_gemv.h"
 #include "kernels_pick.h"
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     float* xs = lds;                      // [D] residual stream of this step
     float* vin = lds + D;                 // [max(D, F)] attention output / FFN hidden
     float* ascr = vin + (F > D ? F : D);  // attention scratch: q, k, v of the head + wave partials
-    int* ptab = reinterpret_cast<int*>(ascr + 192 + kPersistWaves * 68);  // [pages_per_seq]
+    int* ptab = reinterpret_cast<int*>(ascr + 192 + kPersistWaves * 4 * 68);  // [pages_per_seq]
     int tid = threadIdx.x, wave = tid >> 6;
     int lane = tid & 63;
     const int wg = blockIdx.x, G = gridDim.x;
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             if (wg < H) {
                 const int hd = wg;
                 float* qkv = ascr;         // [3][64]: q, key and value of the current position
-                float* part = ascr + 192;  // [waves][68]: m, l, pad, pad, acc[64]
+                float* part = ascr + 192;  // [waves][4 lane groups][68]: m, l, pad, pad, acc[64]
                 const int ctx = pos + 1;
                 // positions are dealt to the wavefronts in runs of `chunk` (a multiple of 4, <= 64)
                 const int chunk = min(64, (((ctx + kPersistWaves - 1) / kPersistWaves) + 3) & ~3);
@@ -505,18 +506,16 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                             k4[it] = reinterpret_cast<const float4*>(qkv + 64)[dl];
                             v4[it] = reinterpret_cast<const float4*>(qkv + 128)[dl];
                         }
-                        float sdot = dot4(q4, k4[it]);
-                        sdot += __shfl_xor(sdot, 1, kWave);
-                        sdot += __shfl_xor(sdot, 2, kWave);
-                        sdot += __shfl_xor(sdot, 4, kWave);
-                        sdot += __shfl_xor(sdot, 8, kWave);
+                        const float sdot = row16_sum(dot4(q4, k4[it]));
                         sc[it] = (in_run && tt < ctx) ? sdot * 0.125f : -INFINITY;  // 1/sqrt(64)
                     }
                     float mb = sc[0];
 #pragma unroll
                     for (int it = 1; it < 8; it++) mb = fmaxf(mb, sc[it]);
-                    mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));
-                    mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
+                    // the four position groups of the wavefront share one running maximum
+                    mb = fmaxf(mb, dpp_move<0x142, 0xA>(mb, mb));
+                    mb = fmaxf(mb, dpp_move<0x143, 0xC>(mb, mb));
+                    mb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mb), 63));
                     const float mn = fmaxf(m, mb);
                     if (mn > -INFINITY) {
                         const float f = expf(m - mn);  // 0 on the first batch (m = -inf)
@@ -537,30 +536,29 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                         m = mn;
                     }
                 }
-                // lsum and acc hold this lane group's share; sum the four groups
-                lsum += __shfl_xor(lsum, 16, kWave);
-                lsum += __shfl_xor(lsum, 32, kWave);
-#pragma unroll
-                for (int o = 16; o < 64; o <<= 1) {
-                    acc.x += __shfl_xor(acc.x, o, kWave);
-                    acc.y += __shfl_xor(acc.y, o, kWave);
-                    acc.z += __shfl_xor(acc.z, o, kWave);
-                    acc.w += __shfl_xor(acc.w, o, kWave);
-                }
-                if (lane < 16) reinterpret_cast<float4*>(part + wave * 68 + 4)[lane] = acc;
-                if (lane == 0) {
-                    part[wave * 68] = m;
-                    part[wave * 68 + 1] = lsum;
+                // every lane group (16 lanes = one position slot) leaves its share; the
+                // groups of a wavefront share its running maximum
+                float* mine = part + (wave * 4 + sub) * 68;
+                reinterpret_cast<float4*>(mine + 4)[dl] = acc;
+                if (dl == 0) {
+                    mine[0] = m;
+                    mine[1] = lsum;
                 }
                 __syncthreads();
                 if (tid < HS) {
                     float M = -INFINITY;
-                    for (int w8 = 0; w8 < kPersistWaves; w8++) M = fmaxf(M, part[w8 * 68]);
+                    for (int w8 = 0; w8 < kPersistWaves; w8++) M = fmaxf(M, part[w8 * 4 * 68]);
                     float Lsum = 0.0f, o = 0.0f;
                     for (int w8 = 0; w8 < kPersistWaves; w8++) {
-                        const float f = expf(part[w8 * 68] - M);  // 0 for wavefronts without positions
-                        Lsum += part[w8 * 68 + 1] * f;
-                        o += part[w8 * 68 + 4 + tid] * f;
+                        const float f = expf(part[w8 * 4 * 68] - M);  // 0 for wavefronts without positions
+                        float ls = 0.0f, os = 0.0f;
+#pragma unroll
+                        for (int g4 = 0; g4 < 4; g4++) {
+                            ls += part[(w8 * 4 + g4) * 68 + 1];
+                            os += part[(w8 * 4 + g4) * 68 + 4 + tid];
+                        }
+                        Lsum += ls * f;
+                        o += os * f;
                     }
                     cell_put(p.at + hd * HS + tid, o * (1.0f / Lsum), tag_of(l, 1));
                 }
