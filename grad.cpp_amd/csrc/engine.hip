@@ -6,6 +6,7 @@
 #include "kernels_attn.h"
 #include "kernels_common.h"
 #include "kernels_gemm.h"
+#include "kernels_gemm_big.h"
 #include "kernels_gemv.h"
 #include "kernels_persist.h"
 #include "kernels_pick.h"
@@ -1030,11 +1031,29 @@ static bool prompt_pass_ok(const Session& s, int len) {
 }
 
 // One projection over M rows (norm folded in for RMSNorm, a norm kernel for LayerNorm).
+// Long row blocks take the compute-bound 128 x 128 tiling, short ones the
+// latency-bound small tiles.
+template <int EPI, bool RMS>
+static void launch_rows_gemm(const GemvParams& g, int M, hipStream_t st) {
+    if (gemm128_ok(g, M)) {
+        static bool lds_raised = false;  // per instantiation: the tile needs more than the default 64 KB
+        if (!lds_raised) {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm128_kernel<EPI, RMS>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          static_cast<int>(kBigLdsBytes)));
+            lds_raised = true;
+        }
+        launch_gemm128<EPI, RMS>(g, M, st);
+    } else {
+        launch_gemm16<EPI, RMS>(g, M, st);
+    }
+}
+
 template <int PRO, int EPI>
 static void project_rows(Session& s, GemvParams g, int M) {
     hipStream_t st = s.stream;
     if (PRO == PRO_RMSNORM) {
-        launch_gemm16<EPI, true>(g, M, st);
+        launch_rows_gemm<EPI, true>(g, M, st);
     } else {
         if (PRO == PRO_LAYERNORM) {
             hipLaunchKernelGGL(norm_rows_kernel, dim3((M + 3) / 4), dim3(256), 0, st, g.in, g.gamma, g.beta,
@@ -1043,7 +1062,7 @@ static void project_rows(Session& s, GemvParams g, int M) {
             g.in = s.pp_norm;
             g.in_stride = g.K;
         }
-        launch_gemm16<EPI, false>(g, M, st);
+        launch_rows_gemm<EPI, false>(g, M, st);
     }
     HIP_CHECK(hipGetLastError());
 }

@@ -1,0 +1,160 @@
+// Projections over many rows (a prompt pass: hundreds to tens of thousands of
+// token rows): C[M,N] = A[M,K] . Wt[N,K]^T on the fp32 matrix cores with the
+// classic compute-bound tiling — one workgroup owns a 128 x 128 tile of C, its
+// four wavefronts 64 x 64 each (16 accumulator tiles of 16 x 16), and A and W
+// travel through LDS in K-steps of 16, double buffered, fetched with
+// row-contiguous 16-byte loads.  The 64-row decode kernel (gemm16_kernel) is
+// bound by latency and wants many small tiles; here the arithmetic is the bound
+// and every fetched element is reused 64 times from LDS.
+//
+// The same prologue and epilogues as the other projection kernels: RMSNorm is
+// folded in (gamma on the way into LDS, the row's sum of squares from the same
+// loads, 1/rms on the finished dot product; layer_norm_row, inference.cpp:33-43)
+// and gemv_epilogue<EPI> consumes column pairs of a row.
+#pragma once
+
+#include "kernels_gemm.h"
+
+namespace gh {
+
+constexpr int kBigTile = 128;       // rows and columns of C per workgroup
+constexpr int kBigK = 16;           // K-step
+constexpr int kBigLd = kBigK + 4;   // LDS row stride of a staged tile (floats): conflict-free float4 access
+constexpr int kBigCLd = kBigTile + 4;  // LDS row stride of the finished tile
+constexpr int kBigThreads = 256;
+constexpr size_t kBigLdsBytes = static_cast<size_t>(kBigTile) * kBigCLd * sizeof(float) + kBigTile * sizeof(float);
+
+template <int EPI, bool RMS>
+__global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p, int M, int n_tiles) {
+    extern __shared__ float lds_big[];
+    // staging: [2 buffers][A | W][128][kBigLd]; after the K loop the same memory
+    // holds the finished tile [128][kBigCLd] and the row scales [128]
+    float* stage = lds_big;
+    float* ctile = lds_big;
+    float* row_scale = lds_big + kBigTile * kBigCLd;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;  // 64 x 64 quadrant of the tile
+    const int j = lane & 15, g = lane >> 4;
+    const int m_tile = blockIdx.x / n_tiles, n_tile = blockIdx.x - m_tile * n_tiles;
+    const int m0 = m_tile * kBigTile, n0 = n_tile * kBigTile;
+    const int K = p.K;
+
+    // fetch assignment: thread t brings rows t/4 and t/4 + 64, 16-byte chunk t%4 of each
+    const int fr = tid >> 2, fc = tid & 3;
+    const float* a_src[2];
+    const float* w_src[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        a_src[h] = p.in + static_cast<size_t>(min(m0 + fr + 64 * h, M - 1)) * p.in_stride + fc * 4;
+        w_src[h] = p.W + static_cast<size_t>(min(n0 + fr + 64 * h, p.N - 1)) * K + fc * 4;
+    }
+    const float* g_src = RMS ? p.gamma + fc * 4 : nullptr;
+
+    v4f acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[a][b] = v4f{0.f, 0.f, 0.f, 0.f};
+    float ss[2] = {0.0f, 0.0f};
+
+    float4 ra[2], rw[2], rg = make_float4(1.f, 1.f, 1.f, 1.f);
+    auto fetch = [&](int k) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            ra[h] = *reinterpret_cast<const float4*>(a_src[h] + k);
+            rw[h] = *reinterpret_cast<const float4*>(w_src[h] + k);
+        }
+        if (RMS) rg = *reinterpret_cast<const float4*>(g_src + k);
+    };
+    auto stash = [&](int buf) {
+        float* as = stage + buf * (2 * kBigTile * kBigLd);
+        float* ws = as + kBigTile * kBigLd;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            float4 a = ra[h];
+            if (RMS) {
+                ss[h] += dot4(a, a);
+                a = make_float4(a.x * rg.x, a.y * rg.y, a.z * rg.z, a.w * rg.w);
+            }
+            *reinterpret_cast<float4*>(as + (fr + 64 * h) * kBigLd + fc * 4) = a;
+            *reinterpret_cast<float4*>(ws + (fr + 64 * h) * kBigLd + fc * 4) = rw[h];
+        }
+    };
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    const int steps = K / kBigK;
+    for (int s = 0; s < steps; s++) {
+        const int buf = s & 1;
+        if (s + 1 < steps) fetch((s + 1) * kBigK);  // in flight while this step multiplies
+        const float* as = stage + buf * (2 * kBigTile * kBigLd) + (wm * 64) * kBigLd;
+        const float* ws = stage + buf * (2 * kBigTile * kBigLd) + kBigTile * kBigLd + (wn * 64) * kBigLd;
+        float4 fa[4], fb[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            fa[t] = *reinterpret_cast<const float4*>(as + (t * 16 + j) * kBigLd + g * 4);
+            fb[t] = *reinterpret_cast<const float4*>(ws + (t * 16 + j) * kBigLd + g * 4);
+        }
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].x, fb[b].x, acc[a][b], 0, 0, 0);
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].y, fb[b].y, acc[a][b], 0, 0, 0);
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].z, fb[b].z, acc[a][b], 0, 0, 0);
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].w, fb[b].w, acc[a][b], 0, 0, 0);
+            }
+        if (s + 1 < steps) stash(buf ^ 1);
+        __syncthreads();
+    }
+
+    // finished tile -> LDS (accumulator layout: lane holds column j, rows 4g + r)
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                ctile[(wm * 64 + a * 16 + 4 * g + r) * kBigCLd + wn * 64 + b * 16 + j] = acc[a][b][r];
+    if (RMS) {
+        // the four threads that fetched a row hold its partial sums of squares
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            float v = ss[h];
+            v += dpp_move<0xB1, 0xF>(v, 0.0f);  // quad_perm [1,0,3,2]
+            v += dpp_move<0x4E, 0xF>(v, 0.0f);  // quad_perm [2,3,0,1]
+            if (fc == 0) row_scale[fr + 64 * h] = 1.0f / sqrtf(v / static_cast<float>(K) + kNormEps);
+        }
+    }
+    __syncthreads();
+    // column pairs (n, n + 1) of one row go through the shared epilogue
+    for (int e = tid; e < kBigTile * (kBigTile / 2); e += kBigThreads) {
+        const int i = e >> 6, jp = (e & 63) * 2;
+        const int m = m0 + i, n = n0 + jp;
+        if (m >= M || n >= p.N) continue;
+        const float2 c = *reinterpret_cast<const float2*>(ctile + i * kBigCLd + jp);
+        float v0 = c.x, v1 = c.y;
+        if (RMS) {
+            const float r = row_scale[i];
+            v0 *= r;
+            v1 *= r;
+        }
+        gemv_epilogue<EPI>(p, m, n, v0, v1, n + 1 < p.N);
+    }
+}
+
+// True when the big-tile kernel applies: enough rows to fill the GPU with
+// 128-row tiles and K a multiple of the K-step.
+inline bool gemm128_ok(const GemvParams& p, int M) {
+    return M >= 4 * kBigTile && p.K % kBigK == 0 && p.in_stride % 4 == 0;
+}
+
+template <int EPI, bool RMS>
+inline void launch_gemm128(const GemvParams& p, int M, hipStream_t st) {
+    const int m_tiles = (M + kBigTile - 1) / kBigTile, n_tiles = (p.N + kBigTile - 1) / kBigTile;
+    hipLaunchKernelGGL((gemm128_kernel<EPI, RMS>), dim3(m_tiles * n_tiles), dim3(kBigThreads), kBigLdsBytes, st, p,
+                       M, n_tiles);
+}
+
+}  // namespace gh
