@@ -41,53 +41,52 @@ __global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p
 
     // fetch assignment: thread t brings rows t/4 and t/4 + 64, 16-byte chunk t%4 of each
     const int fr = tid >> 2, fc = tid & 3;
-    const float* a_src[2];
-    const float* w_src[2];
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        a_src[h] = p.in + static_cast<size_t>(min(m0 + fr + 64 * h, M - 1)) * p.in_stride + fc * 4;
-        w_src[h] = p.W + static_cast<size_t>(min(n0 + fr + 64 * h, p.N - 1)) * K + fc * 4;
-    }
+    const float* a_src0 = p.in + static_cast<size_t>(min(m0 + fr, M - 1)) * p.in_stride + fc * 4;
+    const float* a_src1 = p.in + static_cast<size_t>(min(m0 + fr + 64, M - 1)) * p.in_stride + fc * 4;
+    const float* w_src0 = p.W + static_cast<size_t>(min(n0 + fr, p.N - 1)) * K + fc * 4;
+    const float* w_src1 = p.W + static_cast<size_t>(min(n0 + fr + 64, p.N - 1)) * K + fc * 4;
     const float* g_src = RMS ? p.gamma + fc * 4 : nullptr;
+    const int stash_at = fr * kBigLd + fc * 4;  // this thread's float4 slot in a staged tile (second row: + 64 rows)
 
     v4f acc[4][4];
 #pragma unroll
     for (int a = 0; a < 4; a++)
 #pragma unroll
         for (int b = 0; b < 4; b++) acc[a][b] = v4f{0.f, 0.f, 0.f, 0.f};
-    float ss[2] = {0.0f, 0.0f};
+    float ss0 = 0.0f, ss1 = 0.0f;
 
-    float4 ra[2], rw[2], rg = make_float4(1.f, 1.f, 1.f, 1.f);
-    auto fetch = [&](int k) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            ra[h] = *reinterpret_cast<const float4*>(a_src[h] + k);
-            rw[h] = *reinterpret_cast<const float4*>(w_src[h] + k);
-        }
-        if (RMS) rg = *reinterpret_cast<const float4*>(g_src + k);
-    };
-    auto stash = [&](int buf) {
-        float* as = stage + buf * (2 * kBigTile * kBigLd);
-        float* ws = as + kBigTile * kBigLd;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            float4 a = ra[h];
-            if (RMS) {
-                ss[h] += dot4(a, a);
-                a = make_float4(a.x * rg.x, a.y * rg.y, a.z * rg.z, a.w * rg.w);
-            }
-            *reinterpret_cast<float4*>(as + (fr + 64 * h) * kBigLd + fc * 4) = a;
-            *reinterpret_cast<float4*>(ws + (fr + 64 * h) * kBigLd + fc * 4) = rw[h];
-        }
-    };
+    float4 ra0, ra1, rw0, rw1, rg = make_float4(1.f, 1.f, 1.f, 1.f);
+#define GH_BIG_FETCH(k)                                                  \
+    ra0 = *reinterpret_cast<const float4*>(a_src0 + (k));               \
+    ra1 = *reinterpret_cast<const float4*>(a_src1 + (k));               \
+    rw0 = *reinterpret_cast<const float4*>(w_src0 + (k));               \
+    rw1 = *reinterpret_cast<const float4*>(w_src1 + (k));               \
+    if (RMS) rg = *reinterpret_cast<const float4*>(g_src + (k));
+#define GH_BIG_STASH(buf)                                                                          \
+    {                                                                                              \
+        float* as_ = stage + (buf) * (2 * kBigTile * kBigLd);                                      \
+        float* ws_ = as_ + kBigTile * kBigLd;                                                      \
+        if (RMS) {                                                                                 \
+            ss0 += dot4(ra0, ra0);                                                                 \
+            ss1 += dot4(ra1, ra1);                                                                 \
+            ra0 = make_float4(ra0.x * rg.x, ra0.y * rg.y, ra0.z * rg.z, ra0.w * rg.w);             \
+            ra1 = make_float4(ra1.x * rg.x, ra1.y * rg.y, ra1.z * rg.z, ra1.w * rg.w);             \
+        }                                                                                          \
+        *reinterpret_cast<float4*>(as_ + stash_at) = ra0;                                          \
+        *reinterpret_cast<float4*>(as_ + stash_at + 64 * kBigLd) = ra1;                            \
+        *reinterpret_cast<float4*>(ws_ + stash_at) = rw0;                                          \
+        *reinterpret_cast<float4*>(ws_ + stash_at + 64 * kBigLd) = rw1;                            \
+    }
 
-    fetch(0);
-    stash(0);
+    GH_BIG_FETCH(0)
+    GH_BIG_STASH(0)
     __syncthreads();
     const int steps = K / kBigK;
     for (int s = 0; s < steps; s++) {
         const int buf = s & 1;
-        if (s + 1 < steps) fetch((s + 1) * kBigK);  // in flight while this step multiplies
+        if (s + 1 < steps) {  // in flight while this step multiplies
+            GH_BIG_FETCH((s + 1) * kBigK)
+        }
         const float* as = stage + buf * (2 * kBigTile * kBigLd) + (wm * 64) * kBigLd;
         const float* ws = stage + buf * (2 * kBigTile * kBigLd) + kBigTile * kBigLd + (wn * 64) * kBigLd;
         float4 fa[4], fb[4];
@@ -105,9 +104,11 @@ __global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p
                 acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].z, fb[b].z, acc[a][b], 0, 0, 0);
                 acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].w, fb[b].w, acc[a][b], 0, 0, 0);
             }
-        if (s + 1 < steps) stash(buf ^ 1);
+        if (s + 1 < steps) GH_BIG_STASH(buf ^ 1)
         __syncthreads();
     }
+#undef GH_BIG_FETCH
+#undef GH_BIG_STASH
 
     // finished tile -> LDS (accumulator layout: lane holds column j, rows 4g + r)
 #pragma unroll
@@ -119,12 +120,14 @@ __global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p
                 ctile[(wm * 64 + a * 16 + 4 * g + r) * kBigCLd + wn * 64 + b * 16 + j] = acc[a][b][r];
     if (RMS) {
         // the four threads that fetched a row hold its partial sums of squares
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            float v = ss[h];
-            v += dpp_move<0xB1, 0xF>(v, 0.0f);  // quad_perm [1,0,3,2]
-            v += dpp_move<0x4E, 0xF>(v, 0.0f);  // quad_perm [2,3,0,1]
-            if (fc == 0) row_scale[fr + 64 * h] = 1.0f / sqrtf(v / static_cast<float>(K) + kNormEps);
+        float v0 = ss0, v1 = ss1;
+        v0 += dpp_move<0xB1, 0xF>(v0, 0.0f);  // quad_perm [1,0,3,2]
+        v1 += dpp_move<0xB1, 0xF>(v1, 0.0f);
+        v0 += dpp_move<0x4E, 0xF>(v0, 0.0f);  // quad_perm [2,3,0,1]
+        v1 += dpp_move<0x4E, 0xF>(v1, 0.0f);
+        if (fc == 0) {
+            row_scale[fr] = 1.0f / sqrtf(v0 / static_cast<float>(K) + kNormEps);
+            row_scale[fr + 64] = 1.0f / sqrtf(v1 / static_cast<float>(K) + kNormEps);
         }
     }
     __syncthreads();
