@@ -128,8 +128,8 @@ def main():
         print(json.dumps({"copy_probe_bytes_read": 1 << 30, "copy_probe_bytes_written": 1 << 30}))
         return
     if a.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only (sequences shard across GPUs with no "
-                 "exchange; see DESIGN.md); run with --gpus 1")
+        sys.exit("bench.py: this build runs on one GPU only (more GPUs would each take a share of the "
+                 "sequences, with the weights replicated and nothing exchanged); run with --gpus 1")
 
     import gradhip as G
     from gradhip import synth
