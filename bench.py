@@ -117,7 +117,16 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run a 1 GiB device-to-device copy three times (calibrates rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters against a kernel of known traffic) and exit")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="only time a plain read of 2 GiB (what a streaming kernel can reach of the "
+                         "published HBM peak on this device) and exit")
     a = ap.parse_args()
+    if a.stream_probe:
+        import gradhip as G
+        best = G.read_bandwidth(2 << 30, 5)
+        print(json.dumps({"stream_read_GBps": round(best, 1), "peak_GBps": HBM_PEAK_GBS,
+                          "frac": round(best / HBM_PEAK_GBS, 3)}))
+        return
     if a.copy_probe:
         import torch
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
@@ -185,6 +194,11 @@ def main():
                      "bytes_per_launch": int(bytes_per_launch)},
         "prefill_tok_s": round(r1["prefill_tok_s"], 1),
     }
+    # what a plain streaming-read kernel reaches on this device, measured now: the
+    # practical ceiling the published peak has to be read against
+    stream = G.read_bandwidth(2 << 30, 5)
+    line["roofline"]["stream_read"] = round(stream, 1)
+    line["roofline"]["frac_of_stream_read"] = round(achieved / stream, 4)
 
     if not a.no_batch64:
         greedy = G.sampling(greedy=True, repetition_penalty=1.0)

@@ -1279,6 +1279,27 @@ struct gh_session {
     std::unique_ptr<Session> impl;
 };
 
+// A plain streaming read (eight 16-byte loads in flight per thread): what a
+// bandwidth-bound kernel can reach on this device.
+__global__ __launch_bounds__(256) void stream_read_kernel(const float4* __restrict__ a, size_t n4, float* sink) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    for (; i + 7 * stride < n4; i += 8 * stride) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = a[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            acc.x += v[u].x;
+            acc.y += v[u].y;
+            acc.z += v[u].z;
+            acc.w += v[u].w;
+        }
+    }
+    if (acc.x + acc.y + acc.z + acc.w == 12345.0f) *sink = 1.0f;  // keeps the loads alive
+}
+
 extern "C" {
 
 const char* gh_last_error(void) { return g_last_error.c_str(); }
@@ -1668,6 +1689,38 @@ gh_status gh_device_info(char* name, size_t name_len, int32_t* compute_units, in
         }
         if (compute_units) *compute_units = prop.multiProcessorCount;
         if (is_gfx950) *is_gfx950 = std::strstr(prop.gcnArchName, "gfx950") != nullptr;
+    });
+}
+
+gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per_s) {
+    return guard([&] {
+        require_gpu();
+        if (!gb_per_s || bytes < (1u << 20) || repeats < 1)
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "read bandwidth probe: need >= 1 MiB, >= 1 repeat"};
+        const size_t n4 = bytes / sizeof(float4);
+        float4* buf = nullptr;
+        float* sink = nullptr;
+        HIP_CHECK(hipMalloc(&buf, n4 * sizeof(float4)));
+        HIP_CHECK(hipMalloc(&sink, sizeof(float)));
+        HIP_CHECK(hipMemset(buf, 0, n4 * sizeof(float4)));
+        hipEvent_t e0, e1;
+        HIP_CHECK(hipEventCreate(&e0));
+        HIP_CHECK(hipEventCreate(&e1));
+        double best = 0.0;
+        for (int r = 0; r < repeats + 1; r++) {  // the first pass warms up
+            HIP_CHECK(hipEventRecord(e0, nullptr));
+            hipLaunchKernelGGL(stream_read_kernel, dim3(8192), dim3(256), 0, nullptr, buf, n4, sink);
+            HIP_CHECK(hipEventRecord(e1, nullptr));
+            HIP_CHECK(hipEventSynchronize(e1));
+            float ms = 0.0f;
+            HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+            if (r > 0) best = std::max(best, static_cast<double>(n4) * sizeof(float4) / (ms * 1e-3) / 1e9);
+        }
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        (void)hipFree(buf);
+        (void)hipFree(sink);
+        *gb_per_s = best;
     });
 }
 

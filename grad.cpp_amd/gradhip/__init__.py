@@ -80,6 +80,7 @@ SYMBOLS = {
                                       C.c_uint64, _i32p, _i32p, _f32p, _i32p]),
     "gh_session_last_timing": (C.c_int, [_vp, C.POINTER(GhTiming)]),
     "gh_device_info": (C.c_int, [C.c_char_p, C.c_size_t, _i32p, _i32p]),
+    "gh_device_read_bandwidth": (C.c_int, [C.c_size_t, C.c_int32, C.POINTER(C.c_double)]),
 }
 
 _lib = None
@@ -116,6 +117,13 @@ def device_info():
     cu, ok = C.c_int32(), C.c_int32()
     _check(lib.gh_device_info(name, 256, C.byref(cu), C.byref(ok)))
     return {"name": name.value.decode(), "compute_units": cu.value, "is_gfx950": bool(ok.value)}
+
+
+def read_bandwidth(nbytes: int = 2 << 30, repeats: int = 5) -> float:
+    """GB/s of a plain streaming read of `nbytes` of device memory (best of `repeats`)."""
+    out = C.c_double()
+    _check(load_library().gh_device_read_bandwidth(nbytes, repeats, C.byref(out)))
+    return out.value
 
 
 def _cfg_struct(cfg: synth.Config, fingerprint=None) -> GhConfig:

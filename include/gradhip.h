@@ -213,6 +213,12 @@ gh_status gh_session_last_timing(const gh_session* s, gh_timing* out);
 /* Device facts for reports: name, compute units, and whether it is gfx950. */
 gh_status gh_device_info(char* name, size_t name_len, int32_t* compute_units, int32_t* is_gfx950);
 
+/* Measurement aid with no counterpart in grad.cpp: the rate (GB/s) at which a
+ * plain streaming kernel reads `bytes` of device memory, best of `repeats`
+ * passes.  It says how much of the published HBM peak a bandwidth-bound kernel
+ * can reach on this device, which is what roofline fractions are read against. */
+gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per_s);
+
 #ifdef __cplusplus
 }
 #endif
