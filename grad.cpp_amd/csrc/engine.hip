@@ -659,7 +659,7 @@ static const char* persist_unavailable(const Session& s, int lds_bytes, int cus)
     const Shape& sh = s.m->shape;
     if (s.B != 1) return "the persistent engine decodes one sequence";
     if (!persist_kernel_for(sh)) return "the persistent engine has no kernel for this model shape";
-    if (sh.max_len > 512) return "the persistent engine handles contexts up to 512";
+    if (sh.max_len > 4096) return "the persistent engine handles contexts up to 4096";
     if (s.pick_lds_floats <= 0) return "the vocabulary does not fit the persistent engine's LDS";
     if (cus < sh.heads) return "the GPU has fewer compute units than the model has heads";
     (void)lds_bytes;

@@ -285,7 +285,7 @@ __device__ __forceinline__ void load_qkv_operands(const PersistParams& p, const 
     }
 }
 
-// KD = d_model / 256, KF = FFN width / 256; head size 64; context <= 512.
+// KD = d_model / 256, KF = FFN width / 256; head size 64.
 template <int KD, int KF, bool MODERN>
 __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const PersistParams p) {
     extern __shared__ float lds[];
@@ -425,8 +425,9 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 float* qkv = ascr;         // [3][64]: q, key and value of the current position
                 float* part = ascr + 192;  // [waves][4 lane groups][68]: m, l, pad, pad, acc[64]
                 const int ctx = pos + 1;
-                // positions are dealt to the wavefronts in runs of `chunk` (a multiple of 4, <= 64)
-                const int chunk = min(64, (((ctx + kPersistWaves - 1) / kPersistWaves) + 3) & ~3);
+                // positions are dealt to the wavefronts in runs of `chunk` (a multiple of 4),
+                // walked 32 at a time
+                const int chunk = (((ctx + kPersistWaves - 1) / kPersistWaves) + 3) & ~3;
                 const int sub = lane >> 4, dl = lane & 15;
                 const int t0 = wave * chunk;
                 // Cached rows do not depend on this step's q: the first 32 positions of
@@ -479,16 +480,15 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 const float4 q4 = reinterpret_cast<const float4*>(qkv)[dl];
                 float m = -INFINITY, lsum = 0.0f;
                 float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-                // Two batches of 8 iterations (32 positions); softmax state is merged online.
-                for (int batch = 0; batch < 2; batch++) {
-                    if (batch * 32 >= chunk) break;
-                    if (batch == 1) {
+                // Batches of 8 iterations (32 positions); softmax state is merged online.
+                for (int batch = 0; batch * 32 < chunk; batch++) {
+                    if (batch >= 1) {
 #pragma unroll
                         for (int it = 0; it < 8; it++) {
-                            const int tt = t0 + 32 + it * 4 + sub;
+                            const int tt = t0 + batch * 32 + it * 4 + sub;
                             k4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
                             v4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-                            if (32 + it * 4 < chunk && tt < pos) {
+                            if (batch * 32 + it * 4 < chunk && tt < pos) {
                                 const unsigned ko = static_cast<unsigned>(kv_at(l, 0, hd, tt)) + dl * 4;
                                 const unsigned vo = static_cast<unsigned>(kv_at(l, 1, hd, tt)) + dl * 4;
                                 k4[it] = *reinterpret_cast<const float4*>(pool + ko);

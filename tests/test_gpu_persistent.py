@@ -88,6 +88,27 @@ def test_prefill_then_decode_continues_the_context(models):
     assert int(t.pick(opt, uniforms=[u[0]])[0]) == int(whole[20])
 
 
+def test_long_context_runs_of_more_than_64_positions_per_wavefront():
+    """Beyond 512 positions a wavefront of the attention workgroup walks its run in
+    several passes."""
+    cfg = synth.Config(synth.ARCH_MODERN, 500, 768, 1, 12, 700)
+    W, om = make_pair(cfg, 23, std=0.05, norm_noise=0.1)
+    gm = G.Model.from_tensors(cfg, W)
+    s = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    osess = O.Session(om)
+    toks = synth.uniform_tokens(cfg.max_len, cfg.vocab, 8)
+    for t in toks[:520]:
+        ref = osess.step(int(t))
+    got = s.prefill(toks[None, :520])[0]
+    assert_logits_close(got, ref, 1e-4, "after a 520-token prompt")
+    for i, t in enumerate(toks[520:]):
+        ref = osess.step(int(t))
+        if i % 15 == 0 or i >= len(toks) - 523:
+            assert_logits_close(s.step([int(t)])[0], ref, 1e-4, f"position {520 + i}")
+        else:
+            s.step([int(t)])
+
+
 def test_unsupported_shapes_fall_back_or_refuse(models):
     cfg = synth.Config(synth.ARCH_MODERN, 301, 128, 2, 2, 40)
     gm = G.Model.from_tensors(cfg, synth.make_weights(cfg, 1))
