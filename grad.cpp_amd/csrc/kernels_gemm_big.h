@@ -26,7 +26,7 @@ constexpr size_t kBigLdsBytes = static_cast<size_t>(kBigTile) * kBigCLd * sizeof
 
 template <int EPI, bool RMS>
 __global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p, int M, int n_tiles) {
-    extern __shared__ float lds_big[];
+    extern __shared__ __attribute__((aligned(128))) float lds_big[];
     // staging: [2 buffers][A | W][128][kBigLd]; after the K loop the same memory
     // holds the finished tile [128][kBigCLd] and the row scales [128]
     float* stage = lds_big;

@@ -168,7 +168,7 @@ __device__ inline bool persist_pick(const PersistParams& p, float* lds, int i_pi
     PickParams pk = p.pick;
     pk.n_hist = p.pick.n_hist + i_pick;
     pk.pick_idx = p.pick.pick_idx + i_pick;
-    const int chosen = pick_lds_body(pk, 0, lds, true);
+    const int chosen = pick_lds_body<true>(pk, 0, lds);
     if (tid == 0) {
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         cell_put(p.tokc, __int_as_float(chosen), tok_tag);
@@ -288,7 +288,7 @@ __device__ __forceinline__ void load_qkv_operands(const PersistParams& p, const 
 // KD = d_model / 256, KF = FFN width / 256; head size 64.
 template <int KD, int KF, bool MODERN>
 __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const PersistParams p) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(128))) float lds[];
     constexpr int D = KD * 256, F = KF * 256, HS = 64;
     constexpr int PRO = MODERN ? PRO_RMSNORM : PRO_LAYERNORM;
     constexpr int RL = 8;  // logits rows per wavefront item
@@ -321,22 +321,27 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         return ((run << p.kv.page_shift) + slot) * HS;
     };
 
-    if (p.start_with_pick && p.n_picks > 0) {
-        const unsigned tt = (p.epoch * static_cast<unsigned>(L + 1) + static_cast<unsigned>(L)) * 8u + 6u;
-        if (!persist_pick(p, lds, i_pick, arrive_gen, tt, false)) return;
-        i_pick++;
-        if (wg == 0) {
-            // the pick used the whole LDS; restore the page table
-            __syncthreads();
-            for (int i = tid; i < p.kv.pages_per_seq; i += kPersistThreads) ptab[i] = p.kv.page_table[i];
-            __syncthreads();
-        }
-    }
-
     constexpr int NQKV = 3 * D / 2;  // phase A items: pairs of rows
     const bool has_qkv = wg + G * wave < NQKV;
 
-    for (int s = 0; s < p.n_steps; s++) {
+    for (int s = 0;; s++) {
+        // ===== pick before step s (text_gen.cpp:48-61): the first one of a launch may
+        // use logits that are already in memory, later ones follow step s - 1.  One call
+        // site: the sampler is the largest piece of code in the kernel.
+        if (i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick)) {
+            const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
+                                 + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
+            if (!persist_pick(p, lds, i_pick, arrive_gen, tt, s > 0)) return;
+            i_pick++;
+            if (wg == 0) {
+                // the pick used the whole LDS; restore the page table
+                __syncthreads();
+                for (int i = tid; i < p.kv.pages_per_seq; i += kPersistThreads) ptab[i] = p.kv.page_table[i];
+                __syncthreads();
+            }
+        }
+        stamp();
+        if (s >= p.n_steps) break;
         asm volatile("" : "+v"(tid));  // as in the layer loop below
         wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         lane = tid & 63;
@@ -729,19 +734,6 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         } else {
             // nobody needs this step's logits: the last x stays in its cells
             stamp();
-        }
-        stamp();
-
-        // ===== pick (decode rounds only)
-        if (i_pick < p.n_picks && s >= p.n_prompt - 1) {
-            const unsigned tt = (sb + static_cast<unsigned>(L)) * 8u + 7u;
-            if (!persist_pick(p, lds, i_pick, arrive_gen, tt, true)) return;
-            i_pick++;
-            if (wg == 0) {
-                __syncthreads();
-                for (int i = tid; i < p.kv.pages_per_seq; i += kPersistThreads) ptab[i] = p.kv.page_table[i];
-                __syncthreads();
-            }
         }
         stamp();
     }

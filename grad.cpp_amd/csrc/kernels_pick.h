@@ -121,7 +121,7 @@ __device__ inline void bitonic_desc(float* s, int n2) {
 }
 
 __global__ __launch_bounds__(kPickThreads) void pick_kernel(const PickParams p) {
-    extern __shared__ float lds[];  // sort buffer (sort_cap floats), top-p only
+    extern __shared__ __attribute__((aligned(128))) float lds[];  // sort buffer (sort_cap floats), top-p only
     __shared__ float red[kPickThreads / 64];
     __shared__ int redi[kPickThreads / 64];
     __shared__ unsigned hist256[256];
@@ -826,20 +826,80 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
     return ishare[1];
 }
 
-constexpr int kOrderedWalkLimit = 2048;  // survivors sorted by index and walked by one lane
+// Ordered sums by the whole workgroup: x(0) + x(1) + ... with x(i) >= 0 from
+// get(i).  Every thread adds a contiguous run left to right, the run totals are
+// combined left to right, so the result is the serial sum up to regrouping.
+// parts: one float of LDS per wavefront.  Every thread must call these.
+template <class Get>
+__device__ inline float block_ordered_total(Get get, int n, float* parts) {
+    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+    const int run = (n + nt - 1) / nt;
+    const int lo = min(n, tid * run), hi = min(n, lo + run);
+    float part = 0.0f;
+    for (int i = lo; i < hi; i++) part += get(i);
+    const float wtotal = wave_total_in_order(part, 64);
+    __syncthreads();
+    if (lane == 0) parts[wave] = wtotal;
+    __syncthreads();
+    float total = 0.0f;
+    for (int w = 0; w < nw; w++) total += parts[w];
+    __syncthreads();
+    return total;
+}
+
+// First i in [0, n) whose running sum x(0) + ... + x(i) reaches thr, n when none
+// does.  slot: one int of LDS.
+template <class Get>
+__device__ inline int block_first_reach(Get get, int n, float thr, float* parts, int* slot) {
+    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6;
+    const int run = (n + nt - 1) / nt;
+    const int lo = min(n, tid * run), hi = min(n, lo + run);
+    float part = 0.0f;
+    for (int i = lo; i < hi; i++) part += get(i);
+    // sum of the runs of lower lanes of this wavefront, then of lower wavefronts
+    float before = 0.0f;
+#pragma unroll 8
+    for (int j = 0; j < 64; j++) {
+        const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part), j));
+        before += (j < lane) ? pj : 0.0f;
+    }
+    const float wtotal = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(before + part), 63));
+    __syncthreads();
+    if (lane == 0) parts[wave] = wtotal;
+    if (tid == 0) *slot = n;
+    __syncthreads();
+    float base = 0.0f;
+    for (int w = 0; w < wave; w++) base += parts[w];
+    base += before;
+    if (base < thr) {
+        float cumulative = base;
+        for (int i = lo; i < hi; i++) {
+            cumulative += get(i);
+            if (cumulative >= thr) {
+                atomicMin(slot, i);
+                break;
+            }
+        }
+    }
+    __syncthreads();
+    const int at = *slot;
+    __syncthreads();
+    return at;
+}
+
 
 // The pick for sequence b with the row held in `lds` ([V] values then p.sort_cap
 // floats of sort area).  Every thread of the workgroup must call it; all get the
 // chosen id.  coherent: read the logits with device-scope loads (they were
 // written by other workgroups of the same running kernel).
-__device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool coherent) {
+template <bool coherent>
+__device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
     __shared__ float red[kPickThreads / 64];
     __shared__ int redi[kPickThreads / 64];
     __shared__ unsigned hist256[256];
     __shared__ unsigned bcast[2];
     __shared__ int win_tok[kPenaltyWindow];
     __shared__ int pen_before[64], pen_count[64];
-    __shared__ float fshare[2];
     __shared__ int ishare[2];
 
     const int tid = threadIdx.x, nt = blockDim.x;
@@ -1038,20 +1098,11 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
                 for (int i = S + tid; i < n2; i += nt) srt[i] = -1.0f;
                 __syncthreads();
                 bitonic_desc(srt, n2);
-                if (tid == 0) {
-                    float cumulative = 0.0f;
-                    int cutoff_idx = 0;
-                    for (int i = 0; i < S; i++) {
-                        cumulative += srt[i];
-                        if (cumulative >= p.top_p) {
-                            cutoff_idx = i;
-                            break;
-                        }
-                    }
-                    fshare[0] = srt[cutoff_idx];
-                }
+                // first sorted position whose running sum reaches top_p; never reached:
+                // position 0 (text_gen.cpp:167-177)
+                const int reach = block_first_reach([&](int q) { return srt[q]; }, S, p.top_p, red, &ishare[1]);
+                cutoff = srt[reach < S ? reach : 0];
                 __syncthreads();
-                cutoff = fshare[0];
             }
             int kept = 0;
             for (int i = tid; i < V; i += nt) {
@@ -1063,87 +1114,22 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
         }
         __syncthreads();
 
+        // Renormalise by the index-order total of what is left (text_gen.cpp:178-192) and
+        // walk the cumulative sums in index order (:202-208); cut entries are exact zeros.
+        float* parts = red;
         const bool renorm = p.top_p < 1.0f;
-
-        if (S <= kOrderedWalkLimit && S <= p.sort_cap) {
-            // Few survivors: list their indices, sort ascending, and let one lane
-            // do the exact index-order sums (text_gen.cpp:178-208).
-            int* idx = reinterpret_cast<int*>(srt);
-            int n2 = 1;
-            while (n2 < S) n2 <<= 1;
-            if (tid == 0) ishare[1] = 0;
-            __syncthreads();
-            for (int i = tid; i < V; i += nt)
-                if (val[i] > 0.0f) idx[atomicAdd(&ishare[1], 1)] = i;
-            for (int i = S + tid; i < n2; i += nt) idx[i] = 0x7FFFFFFF;
-            __syncthreads();
-            bitonic_asc_int(idx, n2);
-            if (tid == 0) {
-                float total = 0.0f;
-                if (renorm)
-                    for (int i = 0; i < S; i++) total += val[idx[i]];
-                const bool divide = renorm && total > 0.0f;
-                int pick = V - 1;
-                if (u <= 0.0f) {
-                    pick = 0;
-                } else {
-                    float cumulative = 0.0f;
-                    for (int i = 0; i < S; i++) {
-                        const float pr = val[idx[i]];
-                        cumulative += divide ? pr / total : pr;
-                        if (u <= cumulative) {
-                            pick = idx[i];
-                            break;
-                        }
-                    }
-                }
-                ishare[0] = pick;
-            }
+        float total = 1.0f;
+        bool divide = false;
+        if (renorm) {
+            total = block_ordered_total([&](int q) { return val[q]; }, V, parts);
+            divide = total > 0.0f;
+        }
+        if (u <= 0.0f) {
+            if (tid == 0) ishare[0] = 0;
         } else {
-            // Many survivors: every thread sums a contiguous run of the row in
-            // index order, one lane walks the run totals, then the crossing run.
-            const int run = (V + nt - 1) / nt;
-            const int lo = min(V, tid * run), hi = min(V, lo + run);
-            float part = 0.0f;
-            for (int i = lo; i < hi; i++) part += val[i];
-            float* parts = srt;  // sort area is free again (nt <= sort_cap whenever this path runs)
-            __syncthreads();
-            parts[tid] = part;
-            __syncthreads();
-            if (tid == 0) {
-                float total = 0.0f;
-                if (renorm)
-                    for (int t = 0; t < nt; t++) total += parts[t];
-                const bool divide = renorm && total > 0.0f;
-                int pick = V - 1;
-                if (u <= 0.0f) {
-                    pick = 0;
-                } else {
-                    float cumulative = 0.0f;
-                    for (int t = 0; t < nt; t++) {
-                        const float next = cumulative + (divide ? parts[t] / total : parts[t]);
-                        if (u <= next) {
-                            const int a = min(V, t * run), e = min(V, a + run);
-                            int last = -1;
-                            bool found = false;
-                            for (int i = a; i < e; i++) {
-                                const float pr = val[i];
-                                if (pr > 0.0f) last = i;
-                                cumulative += divide ? pr / total : pr;
-                                if (u <= cumulative && pr > 0.0f) {
-                                    pick = i;
-                                    found = true;
-                                    break;
-                                }
-                            }
-                            if (!found && last >= 0) pick = last;
-                            break;
-                        }
-                        cumulative = next;
-                    }
-                }
-                ishare[0] = pick;
-            }
+            const int at = divide ? block_first_reach([&](int q) { return val[q] / total; }, V, u, parts, &ishare[1])
+                                  : block_first_reach([&](int q) { return val[q]; }, V, u, parts, &ishare[1]);
+            if (tid == 0) ishare[0] = at < V ? at : V - 1;
         }
         __syncthreads();
         chosen = ishare[0];
@@ -1153,9 +1139,9 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds, bool
 }
 
 __global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams p) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(128))) float lds[];
     const int b = blockIdx.x;
-    const int chosen = pick_lds_body(p, b, lds, false);
+    const int chosen = pick_lds_body<false>(p, b, lds);
     if (threadIdx.x == 0) {
         p.hist[static_cast<size_t>(b) * p.hist_stride + p.n_hist] = chosen;  // tokens.push_back(next)
         p.tok[b] = chosen;
