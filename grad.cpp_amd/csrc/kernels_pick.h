@@ -892,6 +892,76 @@ __device__ inline int block_first_reach(Get get, int n, float thr, float* parts,
 // floats of sort area).  Every thread of the workgroup must call it; all get the
 // chosen id.  coherent: read the logits with device-scope loads (they were
 // written by other workgroups of the same running kernel).
+// The top-p cut without sorting (text_gen.cpp:160-177).  The reference sorts the
+// probabilities, adds them in descending order until the sum reaches top_p and
+// cuts below the value found there.  That value is the largest probability c
+// whose upper mass (the sum of everything >= c) reaches top_p, which a bisection
+// over the bit patterns of the (positive) probabilities finds in 31 passes of
+// compare-and-add.  If even the whole mass stays below top_p the reference keeps
+// only the maximum.  NT > 0: the workgroup has NT threads and V <= 32 * NT, so a
+// thread's elements stay in registers across the passes; NT == 0 reads LDS.
+template <int NT>
+__device__ inline float top_p_cutoff(const float* val, int V, float top_p, float* red) {
+    const int tid = threadIdx.x, nt = NT > 0 ? NT : static_cast<int>(blockDim.x);
+    constexpr int ROUNDS = NT > 0 ? 32 : 1;
+    float x[ROUNDS];
+    float pmax = 0.0f;
+    if constexpr (NT > 0) {
+#pragma unroll
+        for (int r = 0; r < ROUNDS; r++) {
+            x[r] = 0.0f;
+            if (r * NT < V) {  // uniform; the last round may read (and discard) floats just past V
+                const float raw = val[r * NT + tid];
+                x[r] = (tid < V - r * NT) ? raw : 0.0f;
+            }
+            pmax = fmaxf(pmax, x[r]);
+        }
+    } else {
+        for (int i = tid; i < V; i += nt) pmax = fmaxf(pmax, val[i]);
+    }
+    pmax = block_max(pmax, red);
+    __shared__ float sums[2][kPickThreads / 64];
+    int calls = 0;
+    auto upper_mass = [&](unsigned key) {
+        const float t = __uint_as_float(key);
+        float mass = 0.0f;
+        if constexpr (NT > 0) {
+#pragma unroll
+            for (int r = 0; r < ROUNDS; r++) mass += (x[r] >= t) ? x[r] : 0.0f;
+        } else {
+            for (int i = tid; i < V; i += nt) {
+                const float v = val[i];
+                mass += (v >= t) ? v : 0.0f;
+            }
+        }
+        // block sum with one barrier per call: successive calls alternate between two
+        // sets of per-wavefront slots
+        const float w = wave_sum(mass);
+        float* slot = sums[calls & 1];
+        calls++;
+        if ((tid & 63) == 0) slot[tid >> 6] = w;
+        __syncthreads();
+        float total = 0.0f;
+        for (int q = 0; q < (nt >> 6); q++) total += slot[q];
+        return total;
+    };
+    const unsigned top = __float_as_uint(pmax);  // bit patterns of positive floats order like the floats
+    if (top < 1u || upper_mass(1u) < top_p) {
+        __syncthreads();
+        return pmax;
+    }
+    // the cut is rarely more than 2^-20 below the maximum: try that as the lower end
+    unsigned lo = 1u, hi = top;
+    if (top > (20u << 23) && upper_mass(top - (20u << 23)) >= top_p) lo = top - (20u << 23);
+    while (lo < hi) {
+        const unsigned mid = lo + (hi - lo + 1u) / 2u;
+        if (upper_mass(mid) >= top_p) lo = mid;
+        else hi = mid - 1u;
+    }
+    __syncthreads();
+    return __uint_as_float(lo);
+}
+
 template <bool coherent>
 __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
     __shared__ float red[kPickThreads / 64];
@@ -1082,28 +1152,10 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
         int S = block_sum_int(nonzero, redi);  // entries with p > 0
 
         if (p.top_p < 1.0f) {
-            float cutoff;
-            if (S > p.sort_cap) {
-                if (tid == 0) *p.err = 1;
-                cutoff = 2.0f;
-            } else {
-                int n2 = 1;
-                while (n2 < S) n2 <<= 1;
-                if (tid == 0) ishare[1] = 0;
-                __syncthreads();
-                for (int i = tid; i < V; i += nt) {
-                    const float v = val[i];
-                    if (v > 0.0f) srt[atomicAdd(&ishare[1], 1)] = v;
-                }
-                for (int i = S + tid; i < n2; i += nt) srt[i] = -1.0f;
-                __syncthreads();
-                bitonic_desc(srt, n2);
-                // first sorted position whose running sum reaches top_p; never reached:
-                // position 0 (text_gen.cpp:167-177)
-                const int reach = block_first_reach([&](int q) { return srt[q]; }, S, p.top_p, red, &ishare[1]);
-                cutoff = srt[reach < S ? reach : 0];
-                __syncthreads();
-            }
+            const bool in_regs = p.sort_cap >= nt;  // a thread may read up to nt floats past V
+            const float cutoff = (nt == 512 && V <= 32 * 512 && in_regs)    ? top_p_cutoff<512>(val, V, p.top_p, red)
+                                 : (nt == 1024 && V <= 32 * 1024 && in_regs) ? top_p_cutoff<1024>(val, V, p.top_p, red)
+                                                                             : top_p_cutoff<0>(val, V, p.top_p, red);
             int kept = 0;
             for (int i = tid; i < V; i += nt) {
                 const float v = val[i];
