@@ -353,33 +353,48 @@ struct PrefillAttnParams {
     float scale;
 };
 
+// Causal attention of a prompt pass on the fp32 matrix cores (head size 64):
+// one workgroup = 64 consecutive queries of one (sequence, head), 16 per
+// wavefront; keys and values of the cache (earlier passes included) stream
+// through LDS in tiles of 64 positions.  Both products are formed transposed,
+//   S^T[key][query] = K . Q^T        O^T[dim][query] += V^T . P^T
+// because the accumulator layout of S^T (a lane holds one query and four
+// consecutive keys) is exactly the B-operand layout the second product needs:
+// the probabilities never leave their registers.  The softmax is the online
+// form (running maximum and sum per query, rescaled when the maximum moves);
+// inference.cpp:211-225 computes the same numbers one query at a time.
+typedef float attn_v4f __attribute__((ext_vector_type(4)));
+
 __global__ __launch_bounds__(256) void attn_prefill64_kernel(const PrefillAttnParams p) {
-    constexpr int HS = 64, TILE = 64, LD = HS + 4;  // padded rows: the 4 keys of a quad hit different banks
-    __shared__ float Ks[TILE * LD];
-    __shared__ float Vs[TILE * LD];
+    constexpr int HS = 64, TILE = 64, LDK = HS + 4, LDV = TILE + 4;  // padded rows: float4 reads of 16 rows hit 64 banks
+    __shared__ float Ks[TILE * LDK];  // [key][dim]
+    __shared__ float Vt[HS * LDV];    // [dim][key]
     const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int tid = threadIdx.x, qi = tid >> 2, c = tid & 3;
-    const int t = qb * TILE + qi;                 // this thread's query (token index in the pass)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 15, g = lane >> 4;
+    const int t = qb * TILE + wave * 16 + j;  // this lane's query (token index in the pass)
     const bool live = t < p.len;
-    const int my_pos = p.pos_base + min(t, p.len - 1);
-    const int last_pos = p.pos_base + min(p.len, qb * TILE + TILE) - 1;  // last key any query here needs
-    float4 q4[16];
+    const int qpos = p.pos_base + min(t, p.len - 1);
+    const int last_pos = p.pos_base + min(p.len, qb * TILE + TILE) - 1;              // last key the workgroup needs
+    const int wave_last = p.pos_base + min(p.len, qb * TILE + wave * 16 + 16) - 1;  // ... and this wavefront
+    // Q^T as the B operand: lane (query j, group g) holds dims 16 * db + 4g .. + 3, pre-scaled
+    float4 qf[4];
     {
         const float* qr = p.q + (static_cast<size_t>(b) * p.len + min(t, p.len - 1)) * p.d_model + h * HS;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const float4 v = reinterpret_cast<const float4*>(qr)[i];
-            q4[i] = make_float4(v.x * p.scale, v.y * p.scale, v.z * p.scale, v.w * p.scale);
+        for (int db = 0; db < 4; db++) {
+            const float4 v = *reinterpret_cast<const float4*>(qr + db * 16 + g * 4);
+            qf[db] = make_float4(v.x * p.scale, v.y * p.scale, v.z * p.scale, v.w * p.scale);
         }
     }
-    float m = -INFINITY, l = 0.0f;
-    float4 o4[16];
+    attn_v4f o[4];  // O^T: lane holds query j, dims 16 * db + 4g + r
 #pragma unroll
-    for (int i = 0; i < 16; i++) o4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int db = 0; db < 4; db++) o[db] = attn_v4f{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.0f;
 
     for (int k0 = 0; k0 <= last_pos; k0 += TILE) {
         __syncthreads();
-        // stage the tile: 64 rows of 16 float4 for K and for V, 4 + 4 loads per thread
+        // stage the tile: K as it is, V transposed; 4 + 4 loads of 16 bytes per thread
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int e = tid + r * 256, row = e >> 4, col = e & 15;
@@ -389,74 +404,82 @@ __global__ __launch_bounds__(256) void attn_prefill64_kernel(const PrefillAttnPa
                 kv4 = *reinterpret_cast<const float4*>(p.kv.pool + kv_offset(p.kv, p.layer, b, 0, h, kp) + col * 4);
                 vv4 = *reinterpret_cast<const float4*>(p.kv.pool + kv_offset(p.kv, p.layer, b, 1, h, kp) + col * 4);
             }
-            *reinterpret_cast<float4*>(&Ks[row * LD + col * 4]) = kv4;
-            *reinterpret_cast<float4*>(&Vs[row * LD + col * 4]) = vv4;
+            *reinterpret_cast<float4*>(&Ks[row * LDK + col * 4]) = kv4;
+            Vt[(col * 4 + 0) * LDV + row] = vv4.x;
+            Vt[(col * 4 + 1) * LDV + row] = vv4.y;
+            Vt[(col * 4 + 2) * LDV + row] = vv4.z;
+            Vt[(col * 4 + 3) * LDV + row] = vv4.w;
         }
         __syncthreads();
-        // scores of this thread's 16 keys of the tile
-        float sc[16];
+        if (k0 > wave_last) continue;  // every key of the tile is in the future of this wavefront's queries
+
+        // S^T: four blocks of 16 keys; lane holds query j, keys k0 + 16 kb + 4g + r
+        attn_v4f sc[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++) {
+            sc[kb] = attn_v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int db = 0; db < 4; db++) {
+                const float4 a = *reinterpret_cast<const float4*>(&Ks[(kb * 16 + j) * LDK + db * 16 + g * 4]);
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, qf[db].x, sc[kb], 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, qf[db].y, sc[kb], 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, qf[db].z, sc[kb], 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, qf[db].w, sc[kb], 0, 0, 0);
+            }
+        }
+        // causal mask (keys up to the query's own position) and the tile's maximum per query
         float mb = -INFINITY;
 #pragma unroll
-        for (int jj = 0; jj < 16; jj++) {
-            const int j = jj * 4 + c;
-            const float* kr = &Ks[j * LD];
-            float s = 0.0f;
+        for (int kb = 0; kb < 4; kb++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) s += dot4(q4[i], *reinterpret_cast<const float4*>(kr + i * 4));
-            sc[jj] = (k0 + j <= my_pos) ? s : -INFINITY;  // causal: keys up to the query's own position
-            mb = fmaxf(mb, sc[jj]);
-        }
-        const float mn = fmaxf(m, mb);
-        if (mn > -INFINITY) {
-            const float f = expf(m - mn);
-            l *= f;
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                o4[i].x *= f;
-                o4[i].y *= f;
-                o4[i].z *= f;
-                o4[i].w *= f;
+            for (int r = 0; r < 4; r++) {
+                const float s = (k0 + kb * 16 + 4 * g + r <= qpos) ? sc[kb][r] : -INFINITY;
+                sc[kb][r] = s;
+                mb = fmaxf(mb, s);
             }
+        mb = fmaxf(mb, __shfl_xor(mb, 16, kWave));  // the four lane groups hold different keys of the same query
+        mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));
+        const float mn = fmaxf(m, mb);  // finite: key 0 is never in the future
+        const float f = expf(m - mn);   // 0 on the first tile
+        float psum = 0.0f;
 #pragma unroll
-            for (int jj = 0; jj < 16; jj++) {
-                const float e = expf(sc[jj] - mn);
-                l += e;
-                const float* vr = &Vs[(jj * 4 + c) * LD];
+        for (int kb = 0; kb < 4; kb++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const float4 v = *reinterpret_cast<const float4*>(vr + i * 4);
-                    o4[i].x += e * v.x;
-                    o4[i].y += e * v.y;
-                    o4[i].z += e * v.z;
-                    o4[i].w += e * v.w;
-                }
+            for (int r = 0; r < 4; r++) {
+                const float e = expf(sc[kb][r] - mn);  // exp(-inf) = 0 for masked keys
+                sc[kb][r] = e;
+                psum += e;
             }
-            m = mn;
+        psum += __shfl_xor(psum, 16, kWave);
+        psum += __shfl_xor(psum, 32, kWave);
+        l = l * f + psum;
+#pragma unroll
+        for (int db = 0; db < 4; db++) {
+            o[db][0] *= f;
+            o[db][1] *= f;
+            o[db][2] *= f;
+            o[db][3] *= f;
         }
+        // O^T += V^T . P^T: K-slot g of step r is key 16 kb + 4g + r on both operands
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+            for (int db = 0; db < 4; db++) {
+                const float4 a = *reinterpret_cast<const float4*>(&Vt[(db * 16 + j) * LDV + kb * 16 + g * 4]);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, sc[kb][0], o[db], 0, 0, 0);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, sc[kb][1], o[db], 0, 0, 0);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, sc[kb][2], o[db], 0, 0, 0);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, sc[kb][3], o[db], 0, 0, 0);
+            }
+        m = mn;
     }
-    // merge the four threads of the query (adjacent lanes)
-    float M = fmaxf(m, dpp_move<0xB1, 0xF>(m, m));
-    M = fmaxf(M, dpp_move<0x4E, 0xF>(M, M));
-    const float f = (m > -INFINITY) ? expf(m - M) : 0.0f;
-    l *= f;
-    l += dpp_move<0xB1, 0xF>(l, 0.0f);
-    l += dpp_move<0x4E, 0xF>(l, 0.0f);
-    const float inv = 1.0f / l;
-    float* orow = p.out + (static_cast<size_t>(b) * p.len + min(t, p.len - 1)) * p.d_model + h * HS;
+    if (live) {
+        const float inv = 1.0f / l;
+        float* orow = p.out + (static_cast<size_t>(b) * p.len + t) * p.d_model + h * HS;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        float4 v = make_float4(o4[i].x * f, o4[i].y * f, o4[i].z * f, o4[i].w * f);
-        v.x += dpp_move<0xB1, 0xF>(v.x, 0.0f);
-        v.y += dpp_move<0xB1, 0xF>(v.y, 0.0f);
-        v.z += dpp_move<0xB1, 0xF>(v.z, 0.0f);
-        v.w += dpp_move<0xB1, 0xF>(v.w, 0.0f);
-        v.x += dpp_move<0x4E, 0xF>(v.x, 0.0f);
-        v.y += dpp_move<0x4E, 0xF>(v.y, 0.0f);
-        v.z += dpp_move<0x4E, 0xF>(v.z, 0.0f);
-        v.w += dpp_move<0x4E, 0xF>(v.w, 0.0f);
-        // thread c of the quad writes dims [16c, 16c + 16)
-        if (live && (i >> 2) == c)
-            reinterpret_cast<float4*>(orow)[i] = make_float4(v.x * inv, v.y * inv, v.z * inv, v.w * inv);
+        for (int db = 0; db < 4; db++)
+            *reinterpret_cast<float4*>(orow + db * 16 + g * 4) =
+                make_float4(o[db][0] * inv, o[db][1] * inv, o[db][2] * inv, o[db][3] * inv);
     }
 }
 
