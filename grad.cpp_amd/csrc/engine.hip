@@ -17,6 +17,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <numeric>
 #include <string>
 #include <vector>
@@ -1036,13 +1037,13 @@ static bool prompt_pass_ok(const Session& s, int len) {
 template <int EPI, bool RMS>
 static void launch_rows_gemm(const GemvParams& g, int M, hipStream_t st) {
     if (gemm128_ok(g, M)) {
-        static bool lds_raised = false;  // per instantiation: the tile needs more than the default 64 KB
-        if (!lds_raised) {
+        // per instantiation, once: the tile needs more than the default 64 KB of LDS
+        static std::once_flag lds_raised;
+        std::call_once(lds_raised, [] {
             HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm128_kernel<EPI, RMS>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize,
                                           static_cast<int>(kBigLdsBytes)));
-            lds_raised = true;
-        }
+        });
         launch_gemm128<EPI, RMS>(g, M, st);
     } else {
         launch_gemm16<EPI, RMS>(g, M, st);
@@ -1698,28 +1699,33 @@ gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per
         if (!gb_per_s || bytes < (1u << 20) || repeats < 1)
             throw ApiError{GH_ERR_INVALID_ARGUMENT, "read bandwidth probe: need >= 1 MiB, >= 1 repeat"};
         const size_t n4 = bytes / sizeof(float4);
-        float4* buf = nullptr;
-        float* sink = nullptr;
-        HIP_CHECK(hipMalloc(&buf, n4 * sizeof(float4)));
-        HIP_CHECK(hipMalloc(&sink, sizeof(float)));
-        HIP_CHECK(hipMemset(buf, 0, n4 * sizeof(float4)));
-        hipEvent_t e0, e1;
-        HIP_CHECK(hipEventCreate(&e0));
-        HIP_CHECK(hipEventCreate(&e1));
+        struct Scratch {  // released on every path out of this function
+            float4* buf = nullptr;
+            float* sink = nullptr;
+            hipEvent_t e0 = nullptr, e1 = nullptr;
+            ~Scratch() {
+                if (e0) (void)hipEventDestroy(e0);
+                if (e1) (void)hipEventDestroy(e1);
+                if (buf) (void)hipFree(buf);
+                if (sink) (void)hipFree(sink);
+            }
+        } t;
+        HIP_CHECK(hipMalloc(&t.buf, n4 * sizeof(float4)));
+        HIP_CHECK(hipMalloc(&t.sink, sizeof(float)));
+        HIP_CHECK(hipMemset(t.buf, 0, n4 * sizeof(float4)));
+        HIP_CHECK(hipEventCreate(&t.e0));
+        HIP_CHECK(hipEventCreate(&t.e1));
         double best = 0.0;
         for (int r = 0; r < repeats + 1; r++) {  // the first pass warms up
-            HIP_CHECK(hipEventRecord(e0, nullptr));
-            hipLaunchKernelGGL(stream_read_kernel, dim3(8192), dim3(256), 0, nullptr, buf, n4, sink);
-            HIP_CHECK(hipEventRecord(e1, nullptr));
-            HIP_CHECK(hipEventSynchronize(e1));
+            HIP_CHECK(hipEventRecord(t.e0, nullptr));
+            hipLaunchKernelGGL(stream_read_kernel, dim3(8192), dim3(256), 0, nullptr, t.buf, n4, t.sink);
+            HIP_CHECK(hipGetLastError());
+            HIP_CHECK(hipEventRecord(t.e1, nullptr));
+            HIP_CHECK(hipEventSynchronize(t.e1));
             float ms = 0.0f;
-            HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+            HIP_CHECK(hipEventElapsedTime(&ms, t.e0, t.e1));
             if (r > 0) best = std::max(best, static_cast<double>(n4) * sizeof(float4) / (ms * 1e-3) / 1e9);
         }
-        (void)hipEventDestroy(e0);
-        (void)hipEventDestroy(e1);
-        (void)hipFree(buf);
-        (void)hipFree(sink);
         *gb_per_s = best;
     });
 }
