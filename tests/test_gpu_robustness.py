@@ -1,0 +1,103 @@
+"""Behaviour around the edges of the session API: interleaved sessions on one
+model, batches that do not fill the 16-row tiles, prompts shorter and longer
+than the one-pass threshold, repeated create/free without leaking device memory."""
+import numpy as np
+import pytest
+
+import gradhip as G
+import oracle_lib as O
+from gradhip import synth
+from helpers import assert_logits_close, lively_std, make_pair
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def llama768():
+    cfg = synth.Config(synth.ARCH_MODERN, 900, 768, 2, 12, 64)
+    W, om = make_pair(cfg, 31, std=0.05, norm_noise=0.1)
+    return cfg, W, om, G.Model.from_tensors(cfg, W)
+
+
+def test_interleaved_sessions_do_not_disturb_each_other(llama768):
+    cfg, W, om, gm = llama768
+    a = G.Session(gm)                                # persistent engine
+    b = G.Session(gm, engine=G.ENGINE_GRAPH)
+    c = G.Session(gm, batch=3)                       # batched kernels
+    oa, ob = O.Session(om), O.Session(om)
+    ta = synth.uniform_tokens(40, cfg.vocab, 1)
+    tb = synth.uniform_tokens(40, cfg.vocab, 2)
+    for i in range(40):
+        ra, rb = oa.step(int(ta[i])), ob.step(int(tb[i]))
+        assert_logits_close(a.step([int(ta[i])])[0], ra, 1e-4, f"a step {i}")
+        lc = c.step([int(ta[i]), int(tb[i]), int(ta[i])])
+        assert_logits_close(b.step([int(tb[i])])[0], rb, 1e-4, f"b step {i}")
+        assert_logits_close(lc[0], ra, 1e-4, f"c[0] step {i}")
+        assert_logits_close(lc[1], rb, 1e-4, f"c[1] step {i}")
+        assert np.array_equal(lc[0], lc[2])
+
+
+@pytest.mark.parametrize("batch", [7, 19, 33, 130])
+def test_batches_that_do_not_fill_a_tile(batch):
+    cfg = synth.Config(synth.ARCH_MODERN, 301, 128, 2, 2, 24)
+    W, om = make_pair(cfg, 5, std=lively_std(cfg), norm_noise=0.1)
+    gm = G.Model.from_tensors(cfg, W)
+    s = G.Session(gm, batch=batch)
+    toks = np.stack([synth.uniform_tokens(12, cfg.vocab, 40, stream=q) for q in range(batch)])
+    last = s.prefill(toks[:, :9])            # one pass (>= 8 tokens)
+    more = [s.step(toks[:, 9 + i]) for i in range(3)]
+    for q in (0, batch // 2, batch - 1):
+        os_ = O.Session(om)
+        for t in toks[q, :9]:
+            ref = os_.step(int(t))
+        assert_logits_close(last[q], ref, 1e-4, f"prompt, sequence {q}")
+        for i in range(3):
+            assert_logits_close(more[i][q], os_.step(int(toks[q, 9 + i])), 1e-4, f"step {i}, sequence {q}")
+
+
+@pytest.mark.parametrize("plen", [1, 3, 7, 8, 9, 31])
+def test_prompts_around_the_one_pass_threshold(llama768, plen):
+    cfg, W, om, gm = llama768
+    toks = synth.uniform_tokens(plen + 2, cfg.vocab, 50 + plen)
+    os_ = O.Session(om)
+    for t in toks[:plen]:
+        ref = os_.step(int(t))
+    for engine in (G.ENGINE_AUTO, G.ENGINE_GRAPH):
+        s = G.Session(gm, engine=engine)
+        assert_logits_close(s.prefill(toks[None, :plen])[0], ref, 1e-4, f"prompt of {plen}, engine {engine}")
+        assert s.position == plen
+        nxt = O.Session(om)
+        for t in toks[:plen + 1]:
+            r2 = nxt.step(int(t))
+        assert_logits_close(s.step([int(toks[plen])])[0], r2, 1e-4, f"step after a prompt of {plen}")
+
+
+def test_sessions_and_models_give_their_memory_back(llama768):
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipDeviceSynchronize() == 0
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    cfg, W, om, gm = llama768
+    toks = synth.uniform_tokens(16, cfg.vocab, 3)
+
+    def cycle():
+        for engine, batch in ((G.ENGINE_AUTO, 1), (G.ENGINE_GRAPH, 1), (G.ENGINE_AUTO, 5)):
+            s = G.Session(gm, batch=batch, engine=engine)
+            s.prefill(np.tile(toks[None, :12], (batch, 1)))
+            s.decode(3, G.sampling(0.8, 40, 0.9, 1.1), seed=1)
+            s.close()
+        m2 = G.Model.from_tensors(cfg, W)
+        G.Session(m2).step([1])
+        del m2
+
+    cycle()
+    free0 = free_bytes()
+    for _ in range(10):
+        cycle()
+    free1 = free_bytes()
+    assert free0 - free1 < 8 << 20, f"{(free0 - free1) >> 20} MiB not returned after 10 create/free cycles"
