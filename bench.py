@@ -167,7 +167,7 @@ def main():
     steps_per_launch = sum(n for n, _, _ in r1["launches"]) / n_l
     achieved = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
     if persistent:
-        kernel = ("gh::persist_decode_kernel<3, 8, true>: one launch = one pick + step round per token "
+        kernel = ("gh::persist_decode_kernel<3, 8, true, true>: one launch = one pick + step round per token "
                   "for a whole run of steps")
     else:
         kernel = "every kernel of the decode round (one launch per fused op), timed as one span"

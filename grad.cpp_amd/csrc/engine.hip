@@ -334,8 +334,8 @@ struct Session {
     int page_shift = 6;
     int pages_per_seq = 0, n_pages = 0;
     int attn_chunk = 64, attn_max_chunks = 1;
-    int sort_cap = 0;
-    int pick_lds_floats = 0;  // > 0: the LDS-resident pick kernel fits (vocab + sort area)
+    bool pick_row_in_lds = false;  // the pick's working row (vocab floats) fits in LDS beside its work area
+    int work_stride = 0;           // floats per sequence of the working rows in global memory
     bool pick_global_scratch = false;
     bool use_prompt_pass = true;
     int launches_per_step = 0;
@@ -349,15 +349,13 @@ struct Session {
     int* page_table = nullptr;
     float *x = nullptr, *h = nullptr, *q = nullptr, *attn = nullptr, *hidden = nullptr,
           *logits = nullptr;
-    float *work = nullptr, *kept_p = nullptr;
-    int* kept_i = nullptr;
+    float* work = nullptr;
     float* attn_part = nullptr;
     unsigned* attn_tickets = nullptr;
     int* tok = nullptr;   // [B] input ids of the next step
     int* hist = nullptr;  // [B][hist_stride]
     int hist_stride = 0;
     DevState* st = nullptr;
-    int* err = nullptr;
     float* uniforms = nullptr;  // device copy for generate
     size_t uniforms_cap = 0;
     float* logit_log = nullptr;  // per-step logits for gh_session_generate
@@ -409,10 +407,9 @@ struct Session {
                         static_cast<void*>(x), static_cast<void*>(h), static_cast<void*>(q),
                         static_cast<void*>(attn), static_cast<void*>(hidden),
                         static_cast<void*>(logits), static_cast<void*>(work),
-                        static_cast<void*>(kept_p), static_cast<void*>(kept_i),
                         static_cast<void*>(attn_part), static_cast<void*>(attn_tickets),
                         static_cast<void*>(tok), static_cast<void*>(hist), static_cast<void*>(st),
-                        static_cast<void*>(err), static_cast<void*>(uniforms),
+                        static_cast<void*>(uniforms),
                         static_cast<void*>(logit_log), static_cast<void*>(cells),
                         static_cast<void*>(ctl), static_cast<void*>(pp_x), static_cast<void*>(pp_q),
                         static_cast<void*>(pp_attn), static_cast<void*>(pp_norm),
@@ -539,7 +536,7 @@ static int enqueue_logits(Session& s) {
 static int enqueue_step(Session& s) {
     const Model& m = *s.m;
     const Shape& sh = m.shape;
-    const int d = sh.d_model, F = sh.d_ff(), V = sh.vocab, B = s.B;
+    const int d = sh.d_model, F = sh.d_ff(), B = s.B;
     const bool modern = sh.modern();
     hipStream_t st = s.stream;
     int launches = 0;
@@ -643,25 +640,29 @@ using PersistKernel = void (*)(const PersistParams);
 
 // The shapes the persistent kernel is built for (head size 64, d_model and FFN
 // width multiples of 256); nullptr for anything else.
-static PersistKernel persist_kernel_for(const Shape& sh) {
+// row_lds: the sampler's working row fits in LDS.
+template <bool ROW_LDS>
+static PersistKernel persist_kernel_of(const Shape& sh) {
     if (sh.head_size() != 64) return nullptr;
     const int d = sh.d_model, F = sh.d_ff();
     if (sh.modern()) {
-        if (d == 768 && F == 2048) return persist_decode_kernel<3, 8, true>;
+        if (d == 768 && F == 2048) return persist_decode_kernel<3, 8, true, ROW_LDS>;
         return nullptr;
     }
-    if (d == 512) return persist_decode_kernel<2, 8, false>;
-    if (d == 768) return persist_decode_kernel<3, 12, false>;
-    if (d == 1024) return persist_decode_kernel<4, 16, false>;
+    if (d == 512) return persist_decode_kernel<2, 8, false, ROW_LDS>;
+    if (d == 768) return persist_decode_kernel<3, 12, false, ROW_LDS>;
+    if (d == 1024) return persist_decode_kernel<4, 16, false, ROW_LDS>;
     return nullptr;
+}
+static PersistKernel persist_kernel_for(const Shape& sh, bool row_lds) {
+    return row_lds ? persist_kernel_of<true>(sh) : persist_kernel_of<false>(sh);
 }
 
 static const char* persist_unavailable(const Session& s, int lds_bytes, int cus) {
     const Shape& sh = s.m->shape;
     if (s.B != 1) return "the persistent engine decodes one sequence";
-    if (!persist_kernel_for(sh)) return "the persistent engine has no kernel for this model shape";
+    if (!persist_kernel_for(sh, s.pick_row_in_lds)) return "the persistent engine has no kernel for this model shape";
     if (sh.max_len > 4096) return "the persistent engine handles contexts up to 4096";
-    if (s.pick_lds_floats <= 0) return "the vocabulary does not fit the persistent engine's LDS";
     if (cus < sh.heads) return "the GPU has fewer compute units than the model has heads";
     (void)lds_bytes;
     return nullptr;
@@ -730,10 +731,11 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     k.u_stride = u_stride;
     k.seed_lo = static_cast<unsigned>(seed & 0xFFFFFFFFu);
     k.seed_hi = static_cast<unsigned>(seed >> 32);
-    k.sort_cap = s.pick_lds_floats - sh.vocab;
-    k.err = s.err;
+    k.work = s.work;
+    k.work_stride = s.work_stride;
+    k.sort_cap = kPickWorkFloats;
 
-    PersistKernel kernel = persist_kernel_for(sh);
+    PersistKernel kernel = persist_kernel_for(sh, s.pick_row_in_lds);
     hipLaunchKernelGGL(kernel, dim3(s.persist_grid), dim3(kPersistThreads), s.persist_lds, s.stream, p);
     HIP_CHECK(hipGetLastError());
 
@@ -856,14 +858,12 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     dev_alloc(s.attn, B * d);
     dev_alloc(s.hidden, B * F);
     dev_alloc(s.logits, B * V);
-    dev_alloc(s.work, B * V);
-    dev_alloc(s.kept_p, B * V);
-    dev_alloc(s.kept_i, B * V);
+    s.work_stride = static_cast<int>((V + kPickThreads + 3) / 4 * 4);
+    dev_alloc(s.work, B * static_cast<size_t>(s.work_stride));
     dev_alloc(s.tok, B);
     s.hist_stride = sh.max_len + 2;
     dev_alloc(s.hist, B * s.hist_stride);
     dev_alloc(s.st, 1);
-    dev_alloc(s.err, 1);
     HIP_CHECK(hipHostMalloc(&s.host_logits, B * V * sizeof(float)));
     HIP_CHECK(hipHostMalloc(&s.host_ids, B * s.hist_stride * sizeof(int)));
     HIP_CHECK(hipHostMalloc(&s.host_err, sizeof(int)));
@@ -880,31 +880,21 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     dev_alloc(s.attn_part, B * sh.heads * s.attn_max_chunks * (sh.head_size() + 2));
     dev_alloc(s.attn_tickets, B * sh.heads);
 
-    // LDS budget of the pick kernels.  The LDS-resident kernel needs the logits
-    // row plus a power-of-two sort area that can hold it; the fallback kernel
-    // sorts in the largest power of two that fits next to its static arrays.
+    // The pick keeps its working row in LDS when vocab floats fit there beside the
+    // work area and the kernel's static arrays; otherwise the row stays in global
+    // memory.
     int dev = 0, lds_bytes = 0;
     HIP_CHECK(hipGetDevice(&dev));
     HIP_CHECK(hipDeviceGetAttribute(&lds_bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
     const size_t reserve = 8192;
-    int cap = 1;
-    while (static_cast<size_t>(cap) * 2 * sizeof(float) + reserve <= static_cast<size_t>(lds_bytes))
-        cap *= 2;
-    s.sort_cap = cap;
-    if (static_cast<size_t>(cap) * sizeof(float) > 48 * 1024) {
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(pick_kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      cap * static_cast<int>(sizeof(float))));
-    }
-    size_t v2 = 1024;
-    while (v2 < V) v2 *= 2;
     s.pick_global_scratch = (o.flags & GH_FLAG_PICK_GLOBAL_SCRATCH) != 0;
     s.use_prompt_pass = (o.flags & GH_FLAG_STEPWISE_PROMPT) == 0;
-    if (!s.pick_global_scratch && (V + v2) * sizeof(float) + reserve <= static_cast<size_t>(lds_bytes)) {
-        s.pick_lds_floats = static_cast<int>(V + v2);
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(pick_lds_kernel),
+    s.pick_row_in_lds = !s.pick_global_scratch
+                        && (V + kPickWorkFloats) * sizeof(float) + reserve <= static_cast<size_t>(lds_bytes);
+    if (s.pick_row_in_lds) {
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(pick_kernel<true>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      s.pick_lds_floats * static_cast<int>(sizeof(float))));
+                                      lds_bytes - static_cast<int>(reserve)));
     }
 
     {
@@ -915,7 +905,8 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
         if (s.engine == GH_ENGINE_AUTO) s.engine = why ? GH_ENGINE_GRAPH : GH_ENGINE_PERSISTENT;
         if (s.engine == GH_ENGINE_PERSISTENT) {
             const size_t work = d + std::max(d, F) + 192 + kPersistWaves * 4 * 68 + s.pages_per_seq;
-            s.persist_lds = std::max(work, static_cast<size_t>(s.pick_lds_floats)) * sizeof(float);
+            const size_t pick = (s.pick_row_in_lds ? V : 0) + kPickWorkFloats;
+            s.persist_lds = std::max(work, pick) * sizeof(float);
             s.persist_grid = std::min(prop.multiProcessorCount, 256);
             dev_alloc(s.cells, 6 * d + F + 1);
             dev_alloc(s.ctl, 1);
@@ -923,7 +914,7 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
                 s.prof_cap = 1 << 16;
                 dev_alloc(s.prof, s.prof_cap);
             }
-            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(persist_kernel_for(sh)),
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(persist_kernel_for(sh, s.pick_row_in_lds)),
                                           hipFuncAttributeMaxDynamicSharedMemorySize,
                                           static_cast<int>(s.persist_lds)));
             s.launches_per_step = 1;
@@ -971,8 +962,6 @@ static void launch_pick(Session& s, const gh_sampling& o, const float* dev_unifo
     PickParams p{};
     p.logits = s.logits;
     p.work = s.work;
-    p.kept_p = s.kept_p;
-    p.kept_i = s.kept_i;
     p.V = s.m->shape.vocab;
     p.hist = s.hist;
     p.hist_stride = s.hist_stride;
@@ -988,16 +977,14 @@ static void launch_pick(Session& s, const gh_sampling& o, const float* dev_unifo
     p.u_stride = u_stride;
     p.seed_lo = static_cast<unsigned>(seed & 0xFFFFFFFFu);
     p.seed_hi = static_cast<unsigned>(seed >> 32);
-    p.sort_cap = s.sort_cap;
-    p.err = s.err;
-    if (s.pick_lds_floats > 0) {
-        p.sort_cap = s.pick_lds_floats - p.V;
-        hipLaunchKernelGGL(pick_lds_kernel, dim3(s.B), dim3(kPickThreads),
-                           static_cast<size_t>(s.pick_lds_floats) * sizeof(float), s.stream, p);
+    p.work_stride = s.work_stride;
+    p.sort_cap = kPickWorkFloats;
+    if (s.pick_row_in_lds) {
+        hipLaunchKernelGGL(pick_kernel<true>, dim3(s.B), dim3(kPickThreads),
+                           static_cast<size_t>(p.V + kPickWorkFloats) * sizeof(float), s.stream, p);
     } else {
-        const bool need_sort = !o.greedy && o.top_p < 1.0f;
-        const size_t lds = need_sort ? static_cast<size_t>(s.sort_cap) * sizeof(float) : 0;
-        hipLaunchKernelGGL(pick_kernel, dim3(s.B), dim3(kPickThreads), lds, s.stream, p);
+        hipLaunchKernelGGL(pick_kernel<false>, dim3(s.B), dim3(kPickThreads), kPickWorkFloats * sizeof(float),
+                           s.stream, p);
     }
     HIP_CHECK(hipGetLastError());
     if (commit) s.n_hist++;
@@ -1009,16 +996,6 @@ static void check_sampling(const gh_sampling& o) {
         throw ApiError{GH_ERR_INVALID_ARGUMENT, "temperature must be positive"};
     if (!(o.repetition_penalty > 0.0f))
         throw ApiError{GH_ERR_INVALID_ARGUMENT, "repetition_penalty must be positive"};
-}
-
-static void check_pick_error(Session& s) {
-    HIP_CHECK(hipMemcpy(s.host_err, s.err, sizeof(int), hipMemcpyDeviceToHost));
-    const int e = *s.host_err;
-    if (e) {
-        HIP_CHECK(hipMemset(s.err, 0, sizeof(int)));
-        throw ApiError{GH_ERR_RUNTIME,
-                       "top-p sampling without top-k needs more LDS than this vocabulary allows"};
-    }
 }
 
 // ---- prompt pass: every prompt token of every sequence through each layer at once
@@ -1557,7 +1534,6 @@ gh_status gh_session_pick(gh_session* sess, const gh_sampling* opt, const float*
         HIP_CHECK(hipMemcpyAsync(s.host_ids, s.tok, s.B * sizeof(int), hipMemcpyDeviceToHost,
                                  s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
-        check_pick_error(s);
         if (out_ids) std::memcpy(out_ids, s.host_ids, s.B * sizeof(int));
     });
 }
@@ -1589,7 +1565,6 @@ gh_status gh_session_decode(gh_session* sess, int32_t max_tokens, const gh_sampl
                                      hipMemcpyDeviceToHost, s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
         check_persist_abort(s);
-        check_pick_error(s);
         if (out_ids)
             for (size_t b = 0; b < B; b++)
                 std::memcpy(out_ids + b * max_tokens, s.host_ids + b * s.hist_stride,
@@ -1654,7 +1629,6 @@ gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t 
                                  hipMemcpyDeviceToHost, s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
         check_persist_abort(s);
-        check_pick_error(s);
         const size_t out_stride = static_cast<size_t>(prompt_len) + max_tokens;
         for (size_t b = 0; b < B; b++)
             std::memcpy(out_tokens + b * out_stride, s.host_ids + b * s.hist_stride,

@@ -128,7 +128,8 @@ __device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float*
 // workgroup's logits rows have landed, picks, records the token in the history
 // and publishes it in the token cell.  The other workgroups return at once and
 // learn the token from the cell.  False: the wait was abandoned.
-__device__ inline bool persist_pick(const PersistParams& p, float* lds, int i_pick,
+template <bool ROW_LDS>
+__device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds, int i_pick,
                                     unsigned arrive_gen, unsigned tok_tag, bool wait_logits) {
     if (blockIdx.x != 0) return true;
     const int tid = threadIdx.x;
@@ -168,7 +169,8 @@ __device__ inline bool persist_pick(const PersistParams& p, float* lds, int i_pi
     PickParams pk = p.pick;
     pk.n_hist = p.pick.n_hist + i_pick;
     pk.pick_idx = p.pick.pick_idx + i_pick;
-    const int chosen = pick_lds_body<true>(pk, 0, lds);
+    const int chosen = ROW_LDS ? pick_body<true, kPersistThreads>(pk, 0, lds, lds + pk.V)
+                               : pick_body<true, kPersistThreads>(pk, 0, pk.work, lds);
     if (tid == 0) {
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         cell_put(p.tokc, __int_as_float(chosen), tok_tag);
@@ -286,7 +288,7 @@ __device__ __forceinline__ void load_qkv_operands(const PersistParams& p, const 
 }
 
 // KD = d_model / 256, KF = FFN width / 256; head size 64.
-template <int KD, int KF, bool MODERN>
+template <int KD, int KF, bool MODERN, bool ROW_LDS>
 __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const PersistParams p) {
     extern __shared__ __attribute__((aligned(128))) float lds[];
     constexpr int D = KD * 256, F = KF * 256, HS = 64;
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         if (i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick)) {
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
-            if (!persist_pick(p, lds, i_pick, arrive_gen, tt, s > 0)) return;
+            if (!persist_pick<ROW_LDS>(p, lds, i_pick, arrive_gen, tt, s > 0)) return;
             i_pick++;
             if (wg == 0) {
                 // the pick used the whole LDS; restore the page table

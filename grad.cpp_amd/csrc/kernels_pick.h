@@ -13,13 +13,11 @@ namespace gh {
 
 constexpr int kPickThreads = 1024;
 constexpr int kPenaltyWindow = 50;  // text_gen.cpp:22
-constexpr int kSeqWalkLimit = 4096; // survivors walked by one lane, in exact index order
 
 struct PickParams {
     const float* logits;  // [batch][V]
-    float* work;          // [batch][V] scratch
-    float* kept_p;        // [batch][V] scratch: surviving probabilities in index order
-    int* kept_i;          // [batch][V] scratch: their indices
+    float* work;          // [batch][work_stride] working rows when they do not fit in LDS
+    int work_stride;      // >= V + kPickThreads (passes may read, and discard, floats past V)
     int V;
     int* hist;  // [batch][hist_stride] token history (prompt + picks)
     int hist_stride;
@@ -34,9 +32,14 @@ struct PickParams {
     const float* uniforms;  // [batch][u_stride] or nullptr
     int u_stride;
     unsigned seed_lo, seed_hi;
-    int sort_cap;  // floats of LDS available for the descending sort (power of two)
-    int* err;      // set to 1 when top-p needs a sort larger than sort_cap
+    int sort_cap;  // floats of LDS work area next to (or instead of) the row
+    int* err;
 };
+
+// LDS work area of the pick: the small-k selection wants two floats per thread
+// and a few more, the fast sampler kFastLdsFloats, and a pass may read up to one
+// float per thread past the end of a row held in LDS.
+constexpr int kPickWorkFloats = 2 * kPickThreads + 64;
 
 __device__ __forceinline__ unsigned mulhi32(unsigned a, unsigned b) { return __umulhi(a, b); }
 
@@ -67,322 +70,46 @@ __device__ __forceinline__ float key_float(unsigned k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
 }
 
-// The k-th largest of v[0..n) (k >= 1), duplicates counted: the value
-// std::sort(descending)[k-1] of text_gen.cpp:145-148.  8-bit radix select.
-__device__ inline float kth_largest(const float* v, int n, int k, unsigned* hist /*256*/,
-                                    unsigned* bcast /*2*/) {
-    unsigned prefix = 0u, mask = 0u;
-    int remaining = k;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0u;
-        __syncthreads();
-        for (int i = threadIdx.x; i < n; i += blockDim.x) {
-            const unsigned key = float_key(v[i]);
-            if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            int left = remaining;
-            int bin = 255;
-            for (; bin > 0; bin--) {
-                if (static_cast<int>(hist[bin]) >= left) break;
-                left -= static_cast<int>(hist[bin]);
-            }
-            bcast[0] = static_cast<unsigned>(bin);
-            bcast[1] = static_cast<unsigned>(left);
-        }
-        __syncthreads();
-        prefix |= bcast[0] << shift;
-        mask |= 255u << shift;
-        remaining = static_cast<int>(bcast[1]);
-        __syncthreads();
-    }
-    return key_float(prefix);
-}
-
-// Descending bitonic sort of s[0..n2), n2 a power of two.
-__device__ inline void bitonic_desc(float* s, int n2) {
-    for (int k = 2; k <= n2; k <<= 1) {
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int i = threadIdx.x; i < n2; i += blockDim.x) {
-                const int ixj = i ^ j;
-                if (ixj > i) {
-                    const float a = s[i], b = s[ixj];
-                    const bool desc = (i & k) == 0;
-                    if (desc ? (a < b) : (a > b)) {
-                        s[i] = b;
-                        s[ixj] = a;
-                    }
-                }
-            }
-            __syncthreads();
-        }
-    }
-}
-
-__global__ __launch_bounds__(kPickThreads) void pick_kernel(const PickParams p) {
-    extern __shared__ __attribute__((aligned(128))) float lds[];  // sort buffer (sort_cap floats), top-p only
-    __shared__ float red[kPickThreads / 64];
-    __shared__ int redi[kPickThreads / 64];
-    __shared__ unsigned hist256[256];
-    __shared__ unsigned bcast[2];
-    __shared__ int win_tok[kPenaltyWindow];
-    __shared__ float fshare[2];
-    __shared__ int ishare[2];
-
-    const int b = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
-    const int V = p.V;
-    const float* logits = p.logits + static_cast<size_t>(b) * V;
-    float* work = p.work + static_cast<size_t>(b) * V;
-    int* hist = p.hist + static_cast<size_t>(b) * p.hist_stride;
-
-    // ---- logits_with_penalty (text_gen.cpp:14-33)
-    for (int i = tid; i < V; i += nt) work[i] = logits[i];
-    const int window = min(kPenaltyWindow, p.n_hist);
-    if (tid < window) win_tok[tid] = hist[p.n_hist - window + tid];
-    __syncthreads();
-    if (p.penalty != 1.0f && tid < window) {
-        const int id = win_tok[tid];
-        bool first = true;
-        for (int e = 0; e < tid; e++) first = first && (win_tok[e] != id);
-        if (first) {
-            int count = 0;
-            for (int e = tid; e < window; e++) count += (win_tok[e] == id);
-            float v = work[id];
-            for (int c = 0; c < count; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
-            work[id] = v;
-        }
-    }
-    __syncthreads();
-
-    int chosen;
-    if (p.greedy) {
-        // First index of the maximum (strict '>' in text_gen.cpp:55-59).
-        float best = -INFINITY;
-        int bi = 0x7FFFFFFF;
-        for (int i = tid; i < V; i += nt) {
-            const float v = work[i];
-            if (v > best) {
-                best = v;
-                bi = i;
-            }
-        }
+// One pass of the workgroup over v[0..n): f(i, v[i]) for i = tid, tid + nt, ...
+// Eight loads are issued before the first use, so a row in global memory costs
+// one memory latency per eight elements of a thread, not one per element.
+// f may store to v[i].
+template <class F>
+__device__ __forceinline__ void row_pass(const float* v, int n, F f) {
+    const int nt = blockDim.x;
+    int i = threadIdx.x;
+    for (; i + 7 * nt < n; i += 8 * nt) {
+        float x[8];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ov = __shfl_xor(best, o, kWave);
-            const int oi = __shfl_xor(bi, o, kWave);
-            if (ov > best || (ov == best && oi < bi)) {
-                best = ov;
-                bi = oi;
-            }
-        }
-        if ((tid & 63) == 0) {
-            red[tid >> 6] = best;
-            redi[tid >> 6] = bi;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            for (int w = 1; w < nt / 64; w++) {
-                if (red[w] > best || (red[w] == best && redi[w] < bi)) {
-                    best = red[w];
-                    bi = redi[w];
-                }
-            }
-            // data[0] seeds the scan in the reference, so an all-NaN or -inf row picks 0.
-            ishare[0] = (bi == 0x7FFFFFFF) ? 0 : bi;
-        }
-        __syncthreads();
-        chosen = ishare[0];
-    } else {
-        // ---- sample_from_logits (text_gen.cpp:135-209)
-        const float inv_t = 1.0f / p.temperature;
-        for (int i = tid; i < V; i += nt) work[i] = work[i] * inv_t;
-        __syncthreads();
-        if (p.top_k > 0 && p.top_k < V) {
-            const float thr = kth_largest(work, V, p.top_k, hist256, bcast);
-            for (int i = tid; i < V; i += nt)
-                if (work[i] < thr) work[i] = -1e10f;
-            __syncthreads();
-        }
-        // Tensor::softmax (tensor.cpp:421-452)
-        float m = -INFINITY;
-        for (int i = tid; i < V; i += nt) m = fmaxf(m, work[i]);
-        m = block_max(m, red);
-        float sum = 0.0f;
-        for (int i = tid; i < V; i += nt) {
-            const float e = expf(work[i] - m);
-            work[i] = e;
-            sum += e;
-        }
-        sum = block_sum(sum, red);
-        const float inv_sum = 1.0f / sum;
-        for (int i = tid; i < V; i += nt) work[i] *= inv_sum;
-        __syncthreads();
-
-        float cutoff = 0.0f;  // keep p >= cutoff; without top-p every entry stays
-        if (p.top_p < 1.0f) {
-            // Sorted-descending cumulative sum until >= top_p (text_gen.cpp:164-177).
-            // Zero probabilities sort last and add nothing, so only the non-zero
-            // entries are sorted.
-            if (tid == 0) ishare[0] = 0;
-            __syncthreads();
-            int mine = 0;
-            for (int i = tid; i < V; i += nt) mine += (work[i] > 0.0f);
-            atomicAdd(&ishare[0], mine);
-            __syncthreads();
-            const int M = ishare[0];
-            __syncthreads();
-            if (M > p.sort_cap) {
-                if (tid == 0) *p.err = 1;
-                cutoff = 2.0f;  // nothing survives; falls through to the V-1 return
-            } else {
-                int n2 = 1;
-                while (n2 < M) n2 <<= 1;
-                if (tid == 0) ishare[1] = 0;
-                __syncthreads();
-                for (int i = tid; i < V; i += nt) {
-                    const float v = work[i];
-                    if (v > 0.0f) lds[atomicAdd(&ishare[1], 1)] = v;
-                }
-                for (int i = M + tid; i < n2; i += nt) lds[i] = -1.0f;
-                __syncthreads();
-                bitonic_desc(lds, n2);
-                if (tid == 0) {
-                    float cumulative = 0.0f;
-                    int cutoff_idx = 0;
-                    for (int i = 0; i < M; i++) {
-                        cumulative += lds[i];
-                        if (cumulative >= p.top_p) {
-                            cutoff_idx = i;
-                            break;
-                        }
-                    }
-                    fshare[0] = lds[cutoff_idx];
-                }
-                __syncthreads();
-                cutoff = fshare[0];
-            }
-        }
-
-        // Survivors (p >= cutoff and p > 0), compacted in index order.
-        float* kp = p.kept_p + static_cast<size_t>(b) * V;
-        int* ki = p.kept_i + static_cast<size_t>(b) * V;
-        const int per = (V + nt - 1) / nt;
-        const int lo = min(V, tid * per), hi = min(V, lo + per);
-        int cnt = 0;
-        for (int i = lo; i < hi; i++) cnt += (work[i] >= cutoff && work[i] > 0.0f);
-        // exclusive scan of cnt over the block
-        __shared__ int scan[kPickThreads];
-        scan[tid] = cnt;
-        __syncthreads();
-        for (int o = 1; o < nt; o <<= 1) {
-            const int v = tid >= o ? scan[tid - o] : 0;
-            __syncthreads();
-            scan[tid] += v;
-            __syncthreads();
-        }
-        int at = scan[tid] - cnt;
-        const int S = scan[nt - 1];
-        for (int i = lo; i < hi; i++) {
-            const float v = work[i];
-            if (v >= cutoff && v > 0.0f) {
-                kp[at] = v;
-                ki[at] = i;
-                at++;
-            }
-        }
-        __syncthreads();
-
-        float u;
-        if (p.uniforms) {
-            u = p.uniforms[static_cast<size_t>(b) * p.u_stride + p.pick_idx];
-        } else {
-            const unsigned w = philox4x32_10(static_cast<unsigned>(p.pick_idx) >> 2,
-                                             static_cast<unsigned>(p.pick_idx) & 3u, p.seed_lo,
-                                             p.seed_hi ^ static_cast<unsigned>(b));
-            u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
-        }
-
-        const bool renorm = p.top_p < 1.0f;
-        if (S <= kSeqWalkLimit) {
-            // One lane, exact index order: total_kept, the division, the walk
-            // (text_gen.cpp:178-208).  Dropped entries are zeros and add nothing.
-            if (tid == 0) {
-                float total = 0.0f;
-                if (renorm)
-                    for (int i = 0; i < S; i++) total += kp[i];
-                const bool divide = renorm && total > 0.0f;
-                int pick = V - 1;
-                if (u <= 0.0f) {
-                    pick = 0;  // `u <= cumulative` already holds at index 0
-                } else {
-                    float cumulative = 0.0f;
-                    for (int i = 0; i < S; i++) {
-                        cumulative += divide ? kp[i] / total : kp[i];
-                        if (u <= cumulative) {
-                            pick = ki[i];
-                            break;
-                        }
-                    }
-                }
-                ishare[0] = pick;
-            }
-        } else {
-            // Many survivors: each thread sums a contiguous run in index order,
-            // one lane walks the run totals and then the run that crosses u.
-            const int run = (S + nt - 1) / nt;
-            const int rlo = min(S, tid * run), rhi = min(S, rlo + run);
-            float part = 0.0f;
-            for (int i = rlo; i < rhi; i++) part += kp[i];
-            float* parts = reinterpret_cast<float*>(scan);
-            __syncthreads();
-            parts[tid] = part;
-            __syncthreads();
-            if (tid == 0) {
-                float total = 0.0f;
-                if (renorm)
-                    for (int t = 0; t < nt; t++) total += parts[t];
-                const bool divide = renorm && total > 0.0f;
-                int pick = V - 1;
-                if (u <= 0.0f) {
-                    pick = 0;
-                } else {
-                    float cumulative = 0.0f;
-                    for (int t = 0; t < nt; t++) {
-                        const float next = cumulative + (divide ? parts[t] / total : parts[t]);
-                        if (u <= next) {
-                            const int a = min(S, t * run), e = min(S, a + run);
-                            for (int i = a; i < e; i++) {
-                                cumulative += divide ? kp[i] / total : kp[i];
-                                if (u <= cumulative) {
-                                    pick = ki[i];
-                                    break;
-                                }
-                            }
-                            if (pick == V - 1 && e > a) pick = ki[e - 1];
-                            break;
-                        }
-                        cumulative = next;
-                    }
-                }
-                ishare[0] = pick;
-            }
-        }
-        __syncthreads();
-        chosen = ishare[0];
+        for (int q = 0; q < 8; q++) x[q] = v[i + q * nt];
+#pragma unroll
+        for (int q = 0; q < 8; q++) f(i + q * nt, x[q]);
     }
+    for (; i < n; i += nt) f(i, v[i]);
+}
 
-    if (tid == 0) {
-        hist[p.n_hist] = chosen;  // tokens.push_back(next_token)
-        p.tok[b] = chosen;
+// f(i, get(i)) for i = lo .. hi - 1 in that order, the values fetched eight at a
+// time; f returns false to stop.
+template <class Get, class F>
+__device__ __forceinline__ void run_pass(Get get, int lo, int hi, F f) {
+    int i = lo;
+    for (; i + 8 <= hi; i += 8) {
+        float x[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) x[q] = get(i + q);
+#pragma unroll
+        for (int q = 0; q < 8; q++)
+            if (!f(i + q, x[q])) return;
     }
+    for (; i < hi; i++)
+        if (!f(i, get(i))) return;
 }
 
 // ---------------------------------------------------------------------------
-// LDS-resident variant: the whole logits row lives in LDS, every pass over it is
-// an LDS pass, and the serial parts (sorted running sum, final walk) touch only
-// the survivors.  Used whenever vocab + its sort area fit in LDS; the kernel
-// above is the fallback for larger vocabularies.
+// The working copy of the logits row ("the row") lives in LDS when vocab plus
+// the work area fit there, in global memory (cached in L2, read and written by
+// this workgroup only) otherwise.  Every pass below goes over the row through a
+// plain pointer; the serial parts touch only the survivors of the cuts.
 
 // Suffix scan of a 256-bin histogram by one wavefront: finds the bin holding the
 // `want`-th largest key and how many keys are wanted inside it.
@@ -457,12 +184,12 @@ __device__ inline float kth_largest_lds(const float* v, int n, int k, unsigned* 
 // least k elements are >= T), the elements >= T are few, and the answer is the
 // k-th largest of those.  Falls back to the radix select when k exceeds the
 // workgroup size or `work` (work_cap floats) cannot hold 2 * blockDim.x + 16.
-__device__ inline float kth_largest_block(const float* v, int n, int k, float* work, int work_cap,
+__device__ __forceinline__ float kth_largest_block(const float* v, int n, int k, float* work, int work_cap,
                                           unsigned* hist, unsigned* bcast, int* ishare) {
     const int tid = threadIdx.x, nt = blockDim.x;
     if (k > nt || work_cap < 2 * nt + 16) return kth_largest_lds(v, n, k, hist, bcast);
     float mx = -INFINITY;
-    for (int i = tid; i < n; i += nt) mx = fmaxf(mx, v[i]);
+    row_pass(v, n, [&](int, float x) { mx = fmaxf(mx, x); });
     work[tid] = mx;
     if (tid == 0) ishare[1] = 0;
     __syncthreads();
@@ -470,13 +197,12 @@ __device__ inline float kth_largest_block(const float* v, int n, int k, float* w
     const float T = kth_largest_lds(work, nt, k, hist, bcast);
     __syncthreads();
     float* cand = work + nt;  // [nt + 16]
-    for (int i = tid; i < n; i += nt) {
-        const float x = v[i];
+    row_pass(v, n, [&](int, float x) {
         if (x >= T) {
             const int slot = atomicAdd(&ishare[1], 1);
             if (slot < nt) cand[slot] = x;
         }
-    }
+    });
     __syncthreads();
     const int c = ishare[1];
     __syncthreads();
@@ -499,44 +225,12 @@ __device__ inline float kth_largest_block(const float* v, int n, int k, float* w
     return __uint_as_float(bcast[0]);
 }
 
-// Ascending bitonic sort of ints, n2 a power of two.
-__device__ inline void bitonic_asc_int(int* s, int n2) {
-    for (int k = 2; k <= n2; k <<= 1) {
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int i = threadIdx.x; i < n2; i += blockDim.x) {
-                const int ixj = i ^ j;
-                if (ixj > i) {
-                    const int a = s[i], b = s[ixj];
-                    const bool asc = (i & k) == 0;
-                    if (asc ? (a > b) : (a < b)) {
-                        s[i] = b;
-                        s[ixj] = a;
-                    }
-                }
-            }
-            __syncthreads();
-        }
-    }
-}
-
-__device__ __forceinline__ int block_sum_int(int v, int* scratch) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-    __syncthreads();
-    if (lane == 0) scratch[wave] = v;
-    __syncthreads();
-    int r = 0;
-    for (int w = 0; w < nw; w++) r += scratch[w];
-    return r;
-}
-
 // The sampler's tail for at most 64 survivors of the top-k cut, run by one
 // wavefront with lane i holding survivor i in index order: softmax, top-p,
 // renormalisation and the inverse-CDF walk (text_gen.cpp:156-208).  Every sum the
 // reference forms in index or sorted order is formed in that same order here
 // (entries cut by top-k are exact zeros there and add nothing).
-__device__ inline int pick_small_wave(const float* val, const int* cidx, int S, float top_p, float u,
+__device__ __forceinline__ int pick_small_wave(const float* val, const int* cidx, int S, float top_p, float u,
                                       int V, float* scratch /* >= 256 floats */) {
     const int lane = threadIdx.x & 63;
     int* sidx = reinterpret_cast<int*>(scratch);  // [64] survivor indices, ascending
@@ -666,13 +360,15 @@ constexpr int kFastLdsFloats = 3 * kFastCandCap + 3 * 64 + 128;
 // order.  One wavefront finishes: every sum the reference forms in index order
 // (softmax denominator, renormalisation, the final walk) or in descending order
 // (top-p) is formed in that order, lane by lane.
-// NT = threads of the workgroup (compile time, so that a thread's elements sit
-// at immediate offsets and stay in registers between the two passes); needs
-// V <= 32 * NT and V + NT floats of readable LDS behind val.
-template <int NT>
+// NT = threads of the workgroup and ROUNDS = elements per thread (compile time,
+// so that a thread's elements sit at immediate offsets and stay in registers
+// between the two passes); needs V <= ROUNDS * NT and V + NT readable floats
+// behind val.
+template <int NT, int ROUNDS>
 __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int k, float top_p, float u,
                                        float* work, float* red, int* ishare) {
-    constexpr int nt = NT, nw = NT / 64, ROUNDS = 32;
+    constexpr int nt = NT, nw = NT / 64;
+    static_assert(ROUNDS <= 64, "one mask bit per element of a thread");
     static_assert(NT >= kFastCandCap, "every candidate needs a thread");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (V > ROUNDS * NT) return -1;
@@ -718,14 +414,14 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
 
     if (!(T > -INFINITY)) return -1;  // some wavefront has fewer than R finite values
     // candidates: values >= T with their indices, in arbitrary slots
-    unsigned mine = 0u;
+    unsigned long long mine = 0ull;
 #pragma unroll
-    for (int r = 0; r < ROUNDS; r++) mine |= static_cast<unsigned>(x[r] >= T) << r;
+    for (int r = 0; r < ROUNDS; r++) mine |= static_cast<unsigned long long>(x[r] >= T) << r;
     if (mine) {
-        int slot = atomicAdd(&ishare[1], __popc(mine));
+        int slot = atomicAdd(&ishare[1], __popcll(mine));
         while (mine) {
-            const int r = __ffs(mine) - 1;
-            mine &= mine - 1u;
+            const int r = __ffsll(static_cast<long long>(mine)) - 1;
+            mine &= mine - 1ull;
             if (slot < kFastCandCap) {
                 const int i = r * nt + tid;
                 cand_v[slot] = val[i] * inv_t;
@@ -836,7 +532,10 @@ __device__ inline float block_ordered_total(Get get, int n, float* parts) {
     const int run = (n + nt - 1) / nt;
     const int lo = min(n, tid * run), hi = min(n, lo + run);
     float part = 0.0f;
-    for (int i = lo; i < hi; i++) part += get(i);
+    run_pass(get, lo, hi, [&](int, float x) {
+        part += x;
+        return true;
+    });
     const float wtotal = wave_total_in_order(part, 64);
     __syncthreads();
     if (lane == 0) parts[wave] = wtotal;
@@ -855,7 +554,10 @@ __device__ inline int block_first_reach(Get get, int n, float thr, float* parts,
     const int run = (n + nt - 1) / nt;
     const int lo = min(n, tid * run), hi = min(n, lo + run);
     float part = 0.0f;
-    for (int i = lo; i < hi; i++) part += get(i);
+    run_pass(get, lo, hi, [&](int, float x) {
+        part += x;
+        return true;
+    });
     // sum of the runs of lower lanes of this wavefront, then of lower wavefronts
     float before = 0.0f;
 #pragma unroll 8
@@ -873,13 +575,14 @@ __device__ inline int block_first_reach(Get get, int n, float thr, float* parts,
     base += before;
     if (base < thr) {
         float cumulative = base;
-        for (int i = lo; i < hi; i++) {
-            cumulative += get(i);
+        run_pass(get, lo, hi, [&](int i, float x) {
+            cumulative += x;
             if (cumulative >= thr) {
                 atomicMin(slot, i);
-                break;
+                return false;
             }
-        }
+            return true;
+        });
     }
     __syncthreads();
     const int at = *slot;
@@ -888,22 +591,18 @@ __device__ inline int block_first_reach(Get get, int n, float thr, float* parts,
 }
 
 
-// The pick for sequence b with the row held in `lds` ([V] values then p.sort_cap
-// floats of sort area).  Every thread of the workgroup must call it; all get the
-// chosen id.  coherent: read the logits with device-scope loads (they were
-// written by other workgroups of the same running kernel).
 // The top-p cut without sorting (text_gen.cpp:160-177).  The reference sorts the
 // probabilities, adds them in descending order until the sum reaches top_p and
 // cuts below the value found there.  That value is the largest probability c
 // whose upper mass (the sum of everything >= c) reaches top_p, which a bisection
 // over the bit patterns of the (positive) probabilities finds in 31 passes of
 // compare-and-add.  If even the whole mass stays below top_p the reference keeps
-// only the maximum.  NT > 0: the workgroup has NT threads and V <= 32 * NT, so a
-// thread's elements stay in registers across the passes; NT == 0 reads LDS.
-template <int NT>
+// only the maximum.  NT > 0: the workgroup has NT threads and V <= ROUNDS * NT,
+// so a thread's elements stay in registers across the passes; NT == 0 reads the
+// row on every pass.
+template <int NT, int ROUNDS>
 __device__ inline float top_p_cutoff(const float* val, int V, float top_p, float* red) {
     const int tid = threadIdx.x, nt = NT > 0 ? NT : static_cast<int>(blockDim.x);
-    constexpr int ROUNDS = NT > 0 ? 32 : 1;
     float x[ROUNDS];
     float pmax = 0.0f;
     if constexpr (NT > 0) {
@@ -917,7 +616,7 @@ __device__ inline float top_p_cutoff(const float* val, int V, float top_p, float
             pmax = fmaxf(pmax, x[r]);
         }
     } else {
-        for (int i = tid; i < V; i += nt) pmax = fmaxf(pmax, val[i]);
+        row_pass(val, V, [&](int, float v) { pmax = fmaxf(pmax, v); });
     }
     pmax = block_max(pmax, red);
     __shared__ float sums[2][kPickThreads / 64];
@@ -929,10 +628,7 @@ __device__ inline float top_p_cutoff(const float* val, int V, float top_p, float
 #pragma unroll
             for (int r = 0; r < ROUNDS; r++) mass += (x[r] >= t) ? x[r] : 0.0f;
         } else {
-            for (int i = tid; i < V; i += nt) {
-                const float v = val[i];
-                mass += (v >= t) ? v : 0.0f;
-            }
+            row_pass(val, V, [&](int, float v) { mass += (v >= t) ? v : 0.0f; });
         }
         // block sum with one barrier per call: successive calls alternate between two
         // sets of per-wavefront slots
@@ -962,8 +658,16 @@ __device__ inline float top_p_cutoff(const float* val, int V, float top_p, float
     return __uint_as_float(lo);
 }
 
-template <bool coherent>
-__device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
+// The pick for sequence b.  val: the working row ([V] floats, LDS or global,
+// with one float per thread readable behind it); srt: p.sort_cap floats of LDS.
+// Every thread of the workgroup must call it; all get the chosen id.
+// coherent: read the logits with device-scope loads (they were written by other
+// workgroups of the same running kernel).
+// NT: threads of the workgroup.
+// Always inlined: each call site knows whether val is LDS or global memory, and
+// the row's loads and stores are compiled for that address space.
+template <bool coherent, int NT>
+__device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val, float* srt) {
     __shared__ float red[kPickThreads / 64];
     __shared__ int redi[kPickThreads / 64];
     __shared__ unsigned hist256[256];
@@ -972,11 +676,10 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
     __shared__ int pen_before[64], pen_count[64];
     __shared__ int ishare[2];
 
-    const int tid = threadIdx.x, nt = blockDim.x;
+    constexpr int nt = NT;
+    const int tid = threadIdx.x;
     const int V = p.V;
     const float* logits = p.logits + static_cast<size_t>(b) * V;
-    float* val = lds;
-    float* srt = lds + V;
     const int* hist = p.hist + static_cast<size_t>(b) * p.hist_stride;
 
     // ---- logits_with_penalty (text_gen.cpp:14-33)
@@ -1009,7 +712,7 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
             }
         }
     } else {
-        for (int i = tid; i < V; i += nt) val[i] = logits[i];
+        row_pass(logits, V, [&](int i, float v) { val[i] = v; });
     }
     if (tid < window) win_tok[tid] = window_token;
     if (tid < 64) {
@@ -1049,13 +752,12 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
     if (p.greedy) {
         float best = -INFINITY;
         int bi = 0x7FFFFFFF;
-        for (int i = tid; i < V; i += nt) {
-            const float v = val[i];
+        row_pass(val, V, [&](int i, float v) {
             if (v > best) {
                 best = v;
                 bi = i;
             }
-        }
+        });
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
             const float ov = __shfl_xor(best, o, kWave);
@@ -1093,15 +795,16 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
                                              p.seed_hi ^ static_cast<unsigned>(b));
             u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
         }
-        if (p.top_k > 0 && p.top_k <= 64 && p.top_k < V && p.sort_cap >= kFastLdsFloats && p.sort_cap >= nt
-            && (nt == 512 || nt == 1024)) {
-            const int c = nt == 512
-                              ? sample_topk_fast<512>(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare)
-                              : sample_topk_fast<1024>(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare);
+        // elements per thread when a thread keeps its share of the row in registers
+        const int per_thread = (V + nt - 1) / nt;
+        if (p.top_k > 0 && p.top_k <= 64 && p.top_k < V && p.sort_cap >= kFastLdsFloats && per_thread <= 64) {
+            const int c = per_thread <= 32
+                              ? sample_topk_fast<NT, 32>(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare)
+                              : sample_topk_fast<NT, 64>(val, V, inv_t, p.top_k, p.top_p, u, srt, red, ishare);
             __syncthreads();
             if (c >= 0) return c;
         }
-        for (int i = tid; i < V; i += nt) val[i] = val[i] * inv_t;
+        row_pass(val, V, [&](int i, float v) { val[i] = v * inv_t; });
         __syncthreads();
         if (p.top_k > 0 && p.top_k < V) {
             const float thr = kth_largest_block(val, V, p.top_k, srt, p.sort_cap, hist256, bcast, ishare);
@@ -1110,12 +813,12 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
             int* cidx = reinterpret_cast<int*>(srt);
             if (tid == 0) ishare[1] = 0;
             __syncthreads();
-            for (int i = tid; i < V; i += nt) {
-                if (val[i] >= thr) {
+            row_pass(val, V, [&](int i, float v) {
+                if (v >= thr) {
                     const int slot = atomicAdd(&ishare[1], 1);
                     if (slot < 64) cidx[slot] = i;
                 }
-            }
+            });
             __syncthreads();
             const int S0 = ishare[1];
             if (S0 <= 64 && p.sort_cap >= 512) {
@@ -1128,41 +831,32 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
                 __syncthreads();
                 return c;
             }
-            for (int i = tid; i < V; i += nt)
-                if (val[i] < thr) val[i] = -1e10f;
+            row_pass(val, V, [&](int i, float v) {
+                if (v < thr) val[i] = -1e10f;
+            });
             __syncthreads();
         }
         float m = -INFINITY;
-        for (int i = tid; i < V; i += nt) m = fmaxf(m, val[i]);
+        row_pass(val, V, [&](int, float v) { m = fmaxf(m, v); });
         m = block_max(m, red);
         float sum = 0.0f;
-        for (int i = tid; i < V; i += nt) {
-            const float e = expf(val[i] - m);
+        row_pass(val, V, [&](int i, float v) {
+            const float e = expf(v - m);
             val[i] = e;
             sum += e;
-        }
+        });
         sum = block_sum(sum, red);
         const float inv_sum = 1.0f / sum;
-        int nonzero = 0;
-        for (int i = tid; i < V; i += nt) {
-            const float pr = val[i] * inv_sum;
-            val[i] = pr;
-            nonzero += (pr > 0.0f);
-        }
-        int S = block_sum_int(nonzero, redi);  // entries with p > 0
+        row_pass(val, V, [&](int i, float v) { val[i] = v * inv_sum; });
 
         if (p.top_p < 1.0f) {
-            const bool in_regs = p.sort_cap >= nt;  // a thread may read up to nt floats past V
-            const float cutoff = (nt == 512 && V <= 32 * 512 && in_regs)    ? top_p_cutoff<512>(val, V, p.top_p, red)
-                                 : (nt == 1024 && V <= 32 * 1024 && in_regs) ? top_p_cutoff<1024>(val, V, p.top_p, red)
-                                                                             : top_p_cutoff<0>(val, V, p.top_p, red);
-            int kept = 0;
-            for (int i = tid; i < V; i += nt) {
-                const float v = val[i];
+            float cutoff;
+            if (per_thread <= 32) cutoff = top_p_cutoff<NT, 32>(val, V, p.top_p, red);
+            else if (per_thread <= 64) cutoff = top_p_cutoff<NT, 64>(val, V, p.top_p, red);
+            else cutoff = top_p_cutoff<0, 1>(val, V, p.top_p, red);
+            row_pass(val, V, [&](int i, float v) {
                 if (v < cutoff) val[i] = 0.0f;
-                else kept += (v > 0.0f);
-            }
-            S = block_sum_int(kept, redi);
+            });
         }
         __syncthreads();
 
@@ -1190,10 +884,15 @@ __device__ inline int pick_lds_body(const PickParams& p, int b, float* lds) {
     return chosen;
 }
 
-__global__ __launch_bounds__(kPickThreads) void pick_lds_kernel(const PickParams p) {
+// ROW_LDS: the working row sits in LDS in front of the work area; otherwise in
+// p.work.
+template <bool ROW_LDS>
+__global__ __launch_bounds__(kPickThreads) void pick_kernel(const PickParams p) {
     extern __shared__ __attribute__((aligned(128))) float lds[];
     const int b = blockIdx.x;
-    const int chosen = pick_lds_body<false>(p, b, lds);
+    const int chosen =
+        ROW_LDS ? pick_body<false, kPickThreads>(p, b, lds, lds + p.V)
+                : pick_body<false, kPickThreads>(p, b, p.work + static_cast<size_t>(b) * p.work_stride, lds);
     if (threadIdx.x == 0) {
         p.hist[static_cast<size_t>(b) * p.hist_stride + p.n_hist] = chosen;  // tokens.push_back(next)
         p.tok[b] = chosen;

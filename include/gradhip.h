@@ -104,7 +104,7 @@ typedef struct gh_session_opts {
 } gh_session_opts;
 
 /* Keep the sampler's working row in global memory even when it would fit in
- * LDS (the path vocabularies above ~16k entries take); for testing that path. */
+ * LDS (the path vocabularies above ~38k entries take); for testing that path. */
 enum { GH_FLAG_PICK_GLOBAL_SCRATCH = 1 };
 
 /* Feed prompts token by token (one step() each, as text_gen.cpp:44-46 does)
