@@ -3,6 +3,7 @@
 // include/gradhip.h.
 #include "../../include/gradhip.h"
 #include "checkpoint.h"
+#include "tokenizer.h"
 #include "kernels_attn.h"
 #include "kernels_common.h"
 #include "kernels_gemm.h"
@@ -1281,6 +1282,106 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const float4* __restri
 extern "C" {
 
 const char* gh_last_error(void) { return g_last_error.c_str(); }
+
+// ---- tokenizer (host only)
+
+struct gh_tokenizer {
+    gh::ByteBpe bpe;
+};
+
+gh_status gh_tokenizer_load(const char* path, gh_tokenizer** out) {
+    return guard([&] {
+        if (!path || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *out = nullptr;
+        if (!is_gtok_file(path))
+            throw ApiError{GH_ERR_RUNTIME, std::string("Tokenizer file ") + path
+                                               + ": a v1 tokenizer cache; only GTOK v2 files are supported"};
+        *out = new gh_tokenizer{ByteBpe::load(path)};
+    });
+}
+
+gh_status gh_tokenizer_from_merges(const int32_t* merges, int32_t n_merges, const char* const* specials,
+                                   const int32_t* special_lens, int32_t n_specials, gh_tokenizer** out) {
+    return guard([&] {
+        if (!out || n_merges < 0 || n_specials < 0 || (n_merges > 0 && !merges)
+            || (n_specials > 0 && (!specials || !special_lens)))
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *out = nullptr;
+        std::vector<ByteBpe::Merge> m;
+        m.reserve(static_cast<size_t>(n_merges));
+        for (int32_t r = 0; r < n_merges; r++) m.emplace_back(merges[2 * r], merges[2 * r + 1]);
+        std::vector<std::string> sp;
+        for (int32_t i = 0; i < n_specials; i++)
+            sp.emplace_back(specials[i], static_cast<size_t>(std::max(special_lens[i], 0)));
+        *out = new gh_tokenizer{ByteBpe(std::move(m), std::move(sp))};
+    });
+}
+
+gh_status gh_tokenizer_save(const gh_tokenizer* t, const char* path) {
+    return guard([&] {
+        if (!t || !path) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        t->bpe.save(path);
+    });
+}
+
+void gh_tokenizer_free(gh_tokenizer* t) { delete t; }
+
+gh_status gh_tokenizer_get_info(const gh_tokenizer* t, gh_tokenizer_info* out) {
+    return guard([&] {
+        if (!t || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        out->kind = ByteBpe::kKind;
+        out->vocab_size = t->bpe.vocab_size();
+        out->eos_id = t->bpe.special_id("<|endoftext|>");
+        out->n_merges = static_cast<int32_t>(t->bpe.merges().size());
+        out->n_specials = static_cast<int32_t>(t->bpe.specials().size());
+        out->fingerprint = t->bpe.fingerprint();
+    });
+}
+
+gh_status gh_tokenizer_special_id(const gh_tokenizer* t, const char* token, size_t len, int32_t* id) {
+    return guard([&] {
+        if (!t || !id || (len > 0 && !token)) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        *id = t->bpe.special_id(std::string_view(token, len));
+    });
+}
+
+gh_status gh_tokenizer_encode(const gh_tokenizer* t, const char* text, size_t len, int32_t with_specials,
+                              int32_t* ids, size_t cap, size_t* n) {
+    return guard([&] {
+        if (!t || !n || (len > 0 && !text) || (cap > 0 && !ids))
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        const std::vector<int> got = t->bpe.encode(std::string_view(text, len), with_specials != 0);
+        *n = got.size();
+        std::copy_n(got.begin(), std::min(cap, got.size()), ids);
+    });
+}
+
+gh_status gh_tokenizer_decode(const gh_tokenizer* t, const int32_t* ids, size_t n, char* out, size_t cap,
+                              size_t* len) {
+    return guard([&] {
+        if (!t || !len || (n > 0 && !ids) || (cap > 0 && !out))
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        const std::string got = t->bpe.decode(ids, n);
+        *len = got.size();
+        std::copy_n(got.begin(), std::min(cap, got.size()), out);
+    });
+}
+
+gh_status gh_pretokenize(const char* text, size_t len, size_t* ends, size_t cap, size_t* n) {
+    return guard([&] {
+        if (!n || (len > 0 && !text) || (cap > 0 && !ends)) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        const std::string_view v(text, len);
+        size_t pieces = 0;
+        for (size_t pos = 0; pos < len;) {
+            pos = pretok::piece_end(v, pos);
+            if (pieces < cap) ends[pieces] = pos;
+            pieces++;
+        }
+        *n = pieces;
+    });
+}
+
+int32_t gh_codepoint_class(uint32_t codepoint) { return pretok::classify(codepoint); }
 
 static Shape shape_of(const gh_config& c) {
     Shape s;

@@ -1,0 +1,498 @@
+// Byte-level BPE tokenizer and GPT-2 pre-tokenizer (host code).  Follows the
+// behaviour of grad.cpp's src/tokenizer/pretokenize.cpp and byte_bpe.cpp; the
+// file format, fingerprint and message texts are the reference's, the
+// algorithms are written for this library.
+#include "tokenizer.h"
+
+#include "unicode_classes.h"
+
+#include <algorithm>
+#include <climits>
+#include <cstring>
+#include <fstream>
+#include <functional>
+#include <iterator>
+#include <queue>
+#include <stdexcept>
+
+namespace gh {
+
+// ---------------------------------------------------------------------------
+// pre-tokenizer
+
+namespace pretok {
+
+CharClass classify(std::uint32_t cp) { return static_cast<CharClass>(unicode::class_of(cp)); }
+
+Scalar scalar_at(std::string_view text, std::size_t pos) {
+    const auto* s = reinterpret_cast<const unsigned char*>(text.data()) + pos;
+    const std::size_t left = text.size() - pos;
+    const unsigned char lead = s[0];
+    if (lead < 0x80) return {lead, 1, classify(lead)};
+    const Scalar bad{lead, 1, kOther};
+    // Sequence length and the allowed range of the second byte: the narrowed
+    // ranges exclude overlong forms (E0, F0), surrogates (ED) and anything past
+    // U+10FFFF (F4).
+    std::uint32_t len;
+    unsigned char lo = 0x80, hi = 0xBF;
+    std::uint32_t cp;
+    if (lead >= 0xC2 && lead <= 0xDF) {
+        len = 2;
+        cp = lead & 0x1Fu;
+    } else if ((lead & 0xF0) == 0xE0) {
+        len = 3;
+        cp = lead & 0x0Fu;
+        if (lead == 0xE0) lo = 0xA0;
+        if (lead == 0xED) hi = 0x9F;
+    } else if (lead >= 0xF0 && lead <= 0xF4) {
+        len = 4;
+        cp = lead & 0x07u;
+        if (lead == 0xF0) lo = 0x90;
+        if (lead == 0xF4) hi = 0x8F;
+    } else {
+        return bad;  // 80..C1 and F5..FF never start a sequence
+    }
+    if (left < len || s[1] < lo || s[1] > hi) return bad;
+    cp = (cp << 6) | (s[1] & 0x3Fu);
+    for (std::uint32_t k = 2; k < len; k++) {
+        if ((s[k] & 0xC0) != 0x80) return bad;
+        cp = (cp << 6) | (s[k] & 0x3Fu);
+    }
+    return {cp, len, classify(cp)};
+}
+
+namespace {
+
+// Length of a contraction ('s 't 'm 'd 're 've 'll, lower case only) at pos, or 0.
+std::size_t contraction_at(std::string_view text, std::size_t pos) {
+    if (text[pos] != '\'' || pos + 1 >= text.size()) return 0;
+    const char a = text[pos + 1];
+    if (a == 's' || a == 't' || a == 'm' || a == 'd') return 2;
+    if (pos + 2 >= text.size()) return 0;
+    const char b = text[pos + 2];
+    if ((a == 'r' && b == 'e') || (a == 'v' && b == 'e') || (a == 'l' && b == 'l')) return 3;
+    return 0;
+}
+
+}  // namespace
+
+std::size_t piece_end(std::string_view text, std::size_t pos) {
+    const std::size_t n = text.size();
+    if (const std::size_t c = contraction_at(text, pos)) return pos + c;
+
+    // A run of one class, which may take one leading space with it.
+    std::size_t at = pos;
+    Scalar head = scalar_at(text, at);
+    if (text[pos] == ' ' && pos + 1 < n) {
+        const Scalar after = scalar_at(text, pos + 1);
+        if (after.cls != kSpace) {
+            head = after;
+            at = pos + 1;
+        }
+    }
+    if (head.cls != kSpace) {
+        std::size_t end = at + head.length;
+        while (end < n) {
+            const Scalar s = scalar_at(text, end);
+            if (s.cls != head.cls) break;
+            end += s.length;
+        }
+        return end;
+    }
+
+    // White space.  `\s+(?!\S)` leaves the last white-space scalar of a run to
+    // the piece that follows when text follows the run; a run of one scalar,
+    // or one that ends the text, is a piece by itself (`\s+`).
+    std::size_t end = pos, last_start = pos, scalars = 0;
+    while (end < n) {
+        const Scalar s = scalar_at(text, end);
+        if (s.cls != kSpace) break;
+        last_start = end;
+        end += s.length;
+        scalars++;
+    }
+    return (end == n || scalars == 1) ? end : last_start;
+}
+
+}  // namespace pretok
+
+// ---------------------------------------------------------------------------
+// little-endian fields and the fingerprint hash
+
+namespace {
+
+void put_u32(std::string& out, std::uint32_t v) {
+    const char b[4] = {static_cast<char>(v), static_cast<char>(v >> 8), static_cast<char>(v >> 16),
+                       static_cast<char>(v >> 24)};
+    out.append(b, 4);
+}
+
+void put_u64(std::string& out, std::uint64_t v) {
+    put_u32(out, static_cast<std::uint32_t>(v));
+    put_u32(out, static_cast<std::uint32_t>(v >> 32));
+}
+
+// Cursor over a file image; every failure names the file and the field
+// (byte_io.h:32-74).
+class Cursor {
+public:
+    Cursor(std::string_view data, const std::string& path) : data_(data), path_(path) {}
+
+    [[noreturn]] void fail(const std::string& why) const {
+        throw std::runtime_error("Tokenizer file " + path_ + ": " + why);
+    }
+    std::string_view take(std::size_t n, const char* what) {
+        if (data_.size() - at_ < n) fail(std::string("truncated reading ") + what);
+        const std::string_view out = data_.substr(at_, n);
+        at_ += n;
+        return out;
+    }
+    std::uint32_t u32(const char* what) {
+        const auto* b = reinterpret_cast<const unsigned char*>(take(4, what).data());
+        return b[0] | (std::uint32_t{b[1]} << 8) | (std::uint32_t{b[2]} << 16) | (std::uint32_t{b[3]} << 24);
+    }
+    std::uint64_t u64(const char* what) {
+        if (data_.size() - at_ < 8) fail(std::string("truncated reading ") + what);
+        const std::uint64_t lo = u32(what);
+        return lo | (std::uint64_t{u32(what)} << 32);
+    }
+    std::size_t remaining() const { return data_.size() - at_; }
+
+private:
+    std::string_view data_;
+    const std::string& path_;
+    std::size_t at_ = 0;
+};
+
+constexpr std::uint32_t kMaxVocab = 1u << 24;    // byte_bpe.cpp:27
+constexpr std::uint32_t kMaxSpecials = 1024;     // byte_bpe.cpp:28
+constexpr std::size_t kMaxSpecialBytes = 1024;   // byte_bpe.h:96
+
+std::uint64_t pair_key(int left, int right) {
+    return (std::uint64_t{static_cast<std::uint32_t>(left)} << 32) | static_cast<std::uint32_t>(right);
+}
+
+std::string slurp(const std::string& path) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) throw std::runtime_error("Failed to open tokenizer file: " + path);
+    std::string data((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    if (f.bad()) throw std::runtime_error("Failed to read tokenizer file: " + path);
+    return data;
+}
+
+}  // namespace
+
+void Fnv1a64::bytes(std::string_view data) {
+    for (const char c : data) h_ = (h_ ^ static_cast<unsigned char>(c)) * 0x100000001b3ULL;
+}
+void Fnv1a64::u32(std::uint32_t v) {
+    std::string b;
+    put_u32(b, v);
+    bytes(b);
+}
+void Fnv1a64::str(std::string_view s) {
+    u32(static_cast<std::uint32_t>(s.size()));
+    bytes(s);
+}
+
+// ---------------------------------------------------------------------------
+// ByteBpe
+
+ByteBpe::ByteBpe(std::vector<Merge> merges, std::vector<std::string> specials)
+    : merges_(std::move(merges)), specials_(std::move(specials)) {
+    // validation order and texts of ByteBpe::rebuild (byte_bpe.cpp:372-421)
+    if (specials_.size() > kMaxSpecials)
+        throw std::invalid_argument("too many special tokens (" + std::to_string(specials_.size()) + ")");
+    for (std::size_t i = 0; i < specials_.size(); i++) {
+        const std::string& s = specials_[i];
+        if (s.empty() || s.size() > kMaxSpecialBytes)
+            throw std::invalid_argument("special token " + std::to_string(i) + " has " + std::to_string(s.size())
+                                        + " bytes; allowed 1 to " + std::to_string(kMaxSpecialBytes));
+        for (std::size_t j = 0; j < i; j++)
+            if (specials_[j] == s) throw std::invalid_argument("special token '" + s + "' is listed twice");
+    }
+    const std::size_t vocab = kByteTokens + merges_.size() + specials_.size();
+    if (vocab > kMaxVocab) throw std::invalid_argument("vocabulary of " + std::to_string(vocab) + " is too large");
+
+    token_bytes_.reserve(vocab);
+    for (int b = 0; b < kByteTokens; b++) token_bytes_.emplace_back(1, static_cast<char>(b));
+    rank_.reserve(merges_.size());
+    for (std::size_t r = 0; r < merges_.size(); r++) {
+        const int left = merges_[r].first, right = merges_[r].second;
+        const int known = kByteTokens + static_cast<int>(r);
+        if (left < 0 || right < 0 || left >= known || right >= known)
+            throw std::invalid_argument("merge " + std::to_string(r) + " joins tokens " + std::to_string(left)
+                                        + " and " + std::to_string(right) + ", which it does not follow");
+        if (!rank_.emplace(pair_key(left, right), static_cast<int>(r)).second)
+            throw std::invalid_argument("merge " + std::to_string(r) + " repeats an earlier merge");
+        token_bytes_.push_back(token_bytes_[left] + token_bytes_[right]);
+    }
+    for (const std::string& s : specials_) token_bytes_.push_back(s);
+
+    // compute_fingerprint (byte_bpe.cpp:333-347)
+    Fnv1a64 h;
+    h.str("grad.tokenizer.bytebpe");
+    h.u32(kFileVersion);
+    h.u32(kPretokenizerId);
+    h.u32(static_cast<std::uint32_t>(specials_.size()));
+    for (const std::string& s : specials_) h.str(s);
+    h.u32(static_cast<std::uint32_t>(merges_.size()));
+    for (const Merge& m : merges_) {
+        h.u32(static_cast<std::uint32_t>(m.first));
+        h.u32(static_cast<std::uint32_t>(m.second));
+    }
+    fingerprint_ = h.value();
+}
+
+int ByteBpe::special_id(std::string_view token) const {
+    for (std::size_t i = 0; i < specials_.size(); i++)
+        if (specials_[i] == token) return kByteTokens + static_cast<int>(merges_.size() + i);
+    return -1;
+}
+
+int ByteBpe::rank_of(int left, int right) const {
+    const auto it = rank_.find(pair_key(left, right));
+    return it == rank_.end() ? INT_MAX : it->second;
+}
+
+// Merges the adjacent pair of lowest rank, leftmost first, until no pair has a
+// rank (byte_bpe.cpp:474-476: this replays the merges in training order).  The
+// symbols stay in one array; rank[i] caches the rank of (sym[i], sym[i+1]) and
+// only the two entries around a merge are recomputed.
+void ByteBpe::merge_piece(std::string_view piece, std::vector<int>& out) const {
+    const std::size_t n = piece.size();
+    if (n > kScanLimit) {
+        merge_long_piece(piece, out);
+        return;
+    }
+    std::vector<int> sym(n), rank(n, INT_MAX);
+    for (std::size_t i = 0; i < n; i++) sym[i] = static_cast<unsigned char>(piece[i]);
+    for (std::size_t i = 0; i + 1 < n; i++) rank[i] = rank_of(sym[i], sym[i + 1]);
+    std::size_t len = n;
+    while (len > 1) {
+        std::size_t best = 0;
+        int best_rank = INT_MAX;
+        for (std::size_t i = 0; i + 1 < len; i++) {
+            if (rank[i] < best_rank) {
+                best_rank = rank[i];
+                best = i;
+            }
+        }
+        if (best_rank == INT_MAX) break;
+        sym[best] = kByteTokens + best_rank;
+        sym.erase(sym.begin() + static_cast<std::ptrdiff_t>(best) + 1);
+        rank.erase(rank.begin() + static_cast<std::ptrdiff_t>(best) + 1);
+        len--;
+        rank[best] = best + 1 < len ? rank_of(sym[best], sym[best + 1]) : INT_MAX;
+        if (best > 0) rank[best - 1] = rank_of(sym[best - 1], sym[best]);
+    }
+    out.insert(out.end(), sym.begin(), sym.begin() + static_cast<std::ptrdiff_t>(len));
+}
+
+// The same result for long pieces in O(n log n): symbols in a doubly linked list
+// over the byte positions, candidate pairs in a min-heap ordered by (rank,
+// position).  A popped candidate is acted on only if both of its symbols are
+// still what they were when it was pushed.
+void ByteBpe::merge_long_piece(std::string_view piece, std::vector<int>& out) const {
+    const std::size_t n = piece.size();
+    struct Pair {
+        int rank;
+        std::uint32_t at;  // position of the left symbol
+        int left, right;
+        bool operator>(const Pair& o) const { return rank != o.rank ? rank > o.rank : at > o.at; }
+    };
+    std::vector<int> sym(n);
+    std::vector<std::uint32_t> nxt(n), prv(n);
+    std::priority_queue<Pair, std::vector<Pair>, std::greater<Pair>> heap;
+    const auto none = static_cast<std::uint32_t>(n);
+    for (std::size_t i = 0; i < n; i++) {
+        sym[i] = static_cast<unsigned char>(piece[i]);
+        nxt[i] = static_cast<std::uint32_t>(i + 1);
+        prv[i] = i == 0 ? none : static_cast<std::uint32_t>(i - 1);
+    }
+    const auto offer = [&](std::uint32_t at) {
+        const std::uint32_t r = nxt[at];
+        if (r >= none) return;
+        const int rank = rank_of(sym[at], sym[r]);
+        if (rank != INT_MAX) heap.push({rank, at, sym[at], sym[r]});
+    };
+    for (std::uint32_t i = 0; i + 1 < none; i++) offer(i);
+    while (!heap.empty()) {
+        const Pair c = heap.top();
+        heap.pop();
+        const std::uint32_t r = nxt[c.at];
+        if (sym[c.at] != c.left || r >= none || sym[r] != c.right) continue;  // stale
+        sym[c.at] = kByteTokens + c.rank;
+        sym[r] = -1;  // a removed position never matches a candidate again
+        nxt[c.at] = nxt[r];
+        if (nxt[r] < none) prv[nxt[r]] = c.at;
+        if (prv[c.at] != none) offer(prv[c.at]);
+        offer(c.at);
+    }
+    for (std::uint32_t i = 0; i < none; i = nxt[i]) out.push_back(sym[i]);
+}
+
+void ByteBpe::encode_plain(std::string_view text, std::vector<int>& out) const {
+    // pieces repeat a lot in natural text: remember what each one became
+    std::unordered_map<std::string_view, std::pair<std::size_t, std::size_t>> seen;
+    std::vector<int> seen_ids;
+    for (std::size_t pos = 0; pos < text.size();) {
+        const std::size_t end = pretok::piece_end(text, pos);
+        const std::string_view piece = text.substr(pos, end - pos);
+        pos = end;
+        if (piece.size() == 1) {
+            out.push_back(static_cast<unsigned char>(piece[0]));
+            continue;
+        }
+        if (const auto hit = seen.find(piece); hit != seen.end()) {
+            out.insert(out.end(), seen_ids.begin() + static_cast<std::ptrdiff_t>(hit->second.first),
+                       seen_ids.begin() + static_cast<std::ptrdiff_t>(hit->second.first + hit->second.second));
+            continue;
+        }
+        const std::size_t before = out.size();
+        merge_piece(piece, out);
+        if (seen.size() >= (std::size_t{1} << 20)) {
+            seen.clear();
+            seen_ids.clear();
+        }
+        seen.emplace(piece, std::make_pair(seen_ids.size(), out.size() - before));
+        seen_ids.insert(seen_ids.end(), out.begin() + static_cast<std::ptrdiff_t>(before), out.end());
+    }
+}
+
+std::vector<int> ByteBpe::encode(std::string_view text, bool with_specials) const {
+    std::vector<int> out;
+    if (!with_specials || specials_.empty()) {
+        encode_plain(text, out);
+        return out;
+    }
+    // Special tokens are taken left to right: the earliest occurrence of any of
+    // them, the longest when two start at the same place (byte_bpe.cpp:60-86).
+    const int first_special = kByteTokens + static_cast<int>(merges_.size());
+    std::vector<std::size_t> next(specials_.size(), 0);
+    std::vector<char> fresh(specials_.size(), 0);
+    std::size_t pos = 0;
+    for (;;) {
+        std::size_t at = std::string_view::npos, len = 0;
+        int which = -1;
+        for (std::size_t i = 0; i < specials_.size(); i++) {
+            if (!fresh[i] || (next[i] != std::string_view::npos && next[i] < pos)) {
+                next[i] = text.find(specials_[i], pos);
+                fresh[i] = 1;
+            }
+            if (next[i] == std::string_view::npos) continue;
+            if (next[i] < at || (next[i] == at && specials_[i].size() > len)) {
+                at = next[i];
+                len = specials_[i].size();
+                which = static_cast<int>(i);
+            }
+        }
+        const std::size_t stop = which < 0 ? text.size() : at;
+        encode_plain(text.substr(pos, stop - pos), out);
+        if (which < 0) break;
+        out.push_back(first_special + which);
+        pos = at + len;
+    }
+    return out;
+}
+
+std::string ByteBpe::decode(const int* ids, std::size_t n) const {
+    std::string out;
+    for (std::size_t i = 0; i < n; i++) {
+        const int id = ids[i];
+        if (id < 0 || static_cast<std::size_t>(id) >= token_bytes_.size())
+            throw std::out_of_range("token id " + std::to_string(id) + " is outside the vocabulary of "
+                                    + std::to_string(token_bytes_.size()));
+        out += token_bytes_[static_cast<std::size_t>(id)];
+    }
+    return out;
+}
+
+std::string ByteBpe::file_image() const {
+    std::string buf = "GTOK";
+    put_u32(buf, kFileVersion);
+    put_u32(buf, kPretokenizerId);
+    put_u32(buf, static_cast<std::uint32_t>(vocab_size()));
+    put_u32(buf, static_cast<std::uint32_t>(merges_.size()));
+    put_u32(buf, static_cast<std::uint32_t>(specials_.size()));
+    for (std::size_t k = 0; k < specials_.size(); k++) {
+        put_u32(buf, static_cast<std::uint32_t>(kByteTokens + merges_.size() + k));
+        put_u32(buf, static_cast<std::uint32_t>(specials_[k].size()));
+        buf += specials_[k];
+    }
+    for (const Merge& m : merges_) {
+        put_u32(buf, static_cast<std::uint32_t>(m.first));
+        put_u32(buf, static_cast<std::uint32_t>(m.second));
+    }
+    put_u64(buf, fingerprint_);
+    return buf;
+}
+
+void ByteBpe::save(const std::string& path) const {
+    const std::string buf = file_image();
+    std::ofstream f(path, std::ios::binary);
+    if (!f) throw std::runtime_error("Failed to open file for saving: " + path);
+    f.write(buf.data(), static_cast<std::streamsize>(buf.size()));
+    f.close();
+    if (!f) throw std::runtime_error("Failed while writing tokenizer file: " + path);
+}
+
+ByteBpe ByteBpe::load(const std::string& path) {
+    const std::string data = slurp(path);
+    Cursor in(data, path);
+    if (in.take(4, "magic") != "GTOK") in.fail("not a GTOK tokenizer file");
+    const std::uint32_t version = in.u32("version");
+    if (version != kFileVersion) in.fail("unsupported version " + std::to_string(version));
+    const std::uint32_t pre = in.u32("pre-tokenizer id");
+    if (pre != kPretokenizerId) in.fail("unknown pre-tokenizer id " + std::to_string(pre));
+    const std::uint32_t vocab = in.u32("vocab size");
+    const std::uint32_t n_merges = in.u32("merge count");
+    const std::uint32_t n_specials = in.u32("special token count");
+    if (vocab > kMaxVocab || n_merges > kMaxVocab || n_specials > kMaxSpecials
+        || std::uint64_t{kByteTokens} + n_merges + n_specials != vocab) {
+        in.fail("implausible header: vocab " + std::to_string(vocab) + ", " + std::to_string(n_merges)
+                + " merges, " + std::to_string(n_specials) + " special tokens");
+    }
+    std::vector<std::string> specials;
+    specials.reserve(n_specials);
+    for (std::uint32_t k = 0; k < n_specials; k++) {
+        const std::uint32_t id = in.u32("special token id");
+        if (id != kByteTokens + n_merges + k)
+            in.fail("special token " + std::to_string(k) + " has id " + std::to_string(id)
+                    + "; special ids follow the merges");
+        const std::uint32_t len = in.u32("special token length");
+        if (len == 0 || len > kMaxSpecialBytes)
+            in.fail("special token " + std::to_string(k) + " has an implausible length (" + std::to_string(len)
+                    + " bytes)");
+        specials.emplace_back(in.take(len, "special token"));
+    }
+    if (in.remaining() / 8 < n_merges) in.fail("truncated reading merges");
+    std::vector<Merge> merges;
+    merges.reserve(n_merges);
+    for (std::uint32_t r = 0; r < n_merges; r++) {
+        const std::uint32_t left = in.u32("merge"), right = in.u32("merge");
+        if (left >= kByteTokens + r || right >= kByteTokens + r)
+            in.fail("merge " + std::to_string(r) + " joins tokens " + std::to_string(left) + " and "
+                    + std::to_string(right) + ", which it does not follow");
+        merges.emplace_back(static_cast<int>(left), static_cast<int>(right));
+    }
+    const std::uint64_t stored = in.u64("fingerprint");
+    if (in.remaining() != 0) in.fail("unexpected bytes after the fingerprint");
+    try {
+        ByteBpe tok(std::move(merges), std::move(specials));
+        if (tok.fingerprint() != stored) in.fail("fingerprint does not match the contents (corrupt file)");
+        return tok;
+    } catch (const std::invalid_argument& e) {
+        in.fail(e.what());
+    }
+}
+
+bool is_gtok_file(const std::string& path) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) throw std::runtime_error("Failed to open tokenizer file: " + path);
+    char magic[4] = {0, 0, 0, 0};
+    f.read(magic, 4);
+    return f.gcount() == 4 && std::memcmp(magic, "GTOK", 4) == 0;
+}
+
+}  // namespace gh

@@ -52,6 +52,11 @@ class GhTiming(C.Structure):
                 ("decode_steps", C.c_int32), ("launches_per_step", C.c_int32)]
 
 
+class GhTokenizerInfo(C.Structure):
+    _fields_ = [("kind", C.c_uint32), ("vocab_size", C.c_int32), ("eos_id", C.c_int32),
+                ("n_merges", C.c_int32), ("n_specials", C.c_int32), ("fingerprint", C.c_uint64)]
+
+
 # Every symbol include/gradhip.h declares: name -> (restype, argtypes)
 _f32p, _i32p, _vp = C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_void_p
 SYMBOLS = {
@@ -79,6 +84,19 @@ SYMBOLS = {
     "gh_session_generate": (C.c_int, [_vp, _i32p, C.c_int32, C.c_int32, C.POINTER(GhSampling), _f32p,
                                       C.c_uint64, _i32p, _i32p, _f32p, _i32p]),
     "gh_session_last_timing": (C.c_int, [_vp, C.POINTER(GhTiming)]),
+    "gh_tokenizer_load": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
+    "gh_tokenizer_from_merges": (C.c_int, [_i32p, C.c_int32, C.POINTER(C.c_char_p), _i32p, C.c_int32,
+                                           C.POINTER(_vp)]),
+    "gh_tokenizer_save": (C.c_int, [_vp, C.c_char_p]),
+    "gh_tokenizer_free": (None, [_vp]),
+    "gh_tokenizer_get_info": (C.c_int, [_vp, C.POINTER(GhTokenizerInfo)]),
+    "gh_tokenizer_special_id": (C.c_int, [_vp, C.c_char_p, C.c_size_t, _i32p]),
+    "gh_tokenizer_encode": (C.c_int, [_vp, C.c_char_p, C.c_size_t, C.c_int32, _i32p, C.c_size_t,
+                                      C.POINTER(C.c_size_t)]),
+    "gh_tokenizer_decode": (C.c_int, [_vp, _i32p, C.c_size_t, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]),
+    "gh_pretokenize": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t), C.c_size_t,
+                                 C.POINTER(C.c_size_t)]),
+    "gh_codepoint_class": (C.c_int32, [C.c_uint32]),
     "gh_device_info": (C.c_int, [C.c_char_p, C.c_size_t, _i32p, _i32p]),
     "gh_device_read_bandwidth": (C.c_int, [C.c_size_t, C.c_int32, C.POINTER(C.c_double)]),
 }
@@ -168,6 +186,93 @@ class Model:
     def close(self):
         if self._h:
             load_library().gh_model_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def pretokenize(text: bytes) -> list:
+    """Pieces of `text` under GPT-2's pattern (stands in for grad::pretok::split)."""
+    lib = load_library()
+    n = C.c_size_t()
+    _check(lib.gh_pretokenize(text, len(text), None, 0, C.byref(n)))
+    ends = (C.c_size_t * max(n.value, 1))()
+    _check(lib.gh_pretokenize(text, len(text), ends, n.value, C.byref(n)))
+    out, pos = [], 0
+    for e in ends[:n.value]:
+        out.append(text[pos:e])
+        pos = e
+    return out
+
+
+def codepoint_class(cp: int) -> int:
+    """0 other, 1 letter, 2 number, 3 white space (grad::pretok::classify)."""
+    return load_library().gh_codepoint_class(cp)
+
+
+class Tokenizer:
+    """Byte-level BPE over a GTOK v2 file (stands in for grad::ByteBpe behind grad::Tokenizer).
+    Text goes in and out as bytes: decode(encode(b)) == b for every byte string."""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    @classmethod
+    def load(cls, path) -> "Tokenizer":
+        h = _vp()
+        _check(load_library().gh_tokenizer_load(os.fsencode(path), C.byref(h)))
+        return cls(h.value)
+
+    @classmethod
+    def from_merges(cls, merges, specials=(b"<|endoftext|>",)) -> "Tokenizer":
+        m = np.ascontiguousarray(np.asarray(merges, dtype=np.int32).reshape(-1, 2))
+        sp = [bytes(x) for x in specials]
+        arr = (C.c_char_p * max(len(sp), 1))(*sp)
+        lens = (C.c_int32 * max(len(sp), 1))(*[len(x) for x in sp])
+        h = _vp()
+        _check(load_library().gh_tokenizer_from_merges(m.ctypes.data_as(_i32p), len(m), arr, lens, len(sp),
+                                                       C.byref(h)))
+        return cls(h.value)
+
+    def save(self, path) -> None:
+        _check(load_library().gh_tokenizer_save(self._h, os.fsencode(path)))
+
+    @property
+    def info(self) -> GhTokenizerInfo:
+        out = GhTokenizerInfo()
+        _check(load_library().gh_tokenizer_get_info(self._h, C.byref(out)))
+        return out
+
+    def special_id(self, token: bytes):
+        out = C.c_int32()
+        _check(load_library().gh_tokenizer_special_id(self._h, token, len(token), C.byref(out)))
+        return None if out.value < 0 else out.value
+
+    def encode(self, text: bytes, with_specials=True) -> np.ndarray:
+        lib = load_library()
+        n = C.c_size_t()
+        cap = max(len(text), 1)  # never more ids than bytes
+        ids = np.empty(cap, np.int32)
+        _check(lib.gh_tokenizer_encode(self._h, text, len(text), 1 if with_specials else 0,
+                                       ids.ctypes.data_as(_i32p), cap, C.byref(n)))
+        return ids[:n.value].copy()
+
+    def decode(self, ids) -> bytes:
+        lib = load_library()
+        a = np.ascontiguousarray(ids, dtype=np.int32)
+        n = C.c_size_t()
+        _check(lib.gh_tokenizer_decode(self._h, a.ctypes.data_as(_i32p), len(a), None, 0, C.byref(n)))
+        buf = C.create_string_buffer(max(n.value, 1))
+        _check(lib.gh_tokenizer_decode(self._h, a.ctypes.data_as(_i32p), len(a), buf, n.value, C.byref(n)))
+        return buf.raw[:n.value]
+
+    def close(self):
+        if self._h:
+            load_library().gh_tokenizer_free(self._h)
             self._h = None
 
     def __del__(self):

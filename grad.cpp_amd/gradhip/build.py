@@ -18,7 +18,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-fno-fast-math", "-Wall", "-Wno-unused-function",
 ]
-SOURCES = ["engine.hip", "checkpoint.cpp"]
+SOURCES = ["engine.hip", "checkpoint.cpp", "tokenizer.cpp"]
 
 
 def build(verbose: bool = True) -> str:

@@ -197,6 +197,54 @@ gh_status gh_session_generate(gh_session* s, const int32_t* prompts, int32_t pro
                               uint64_t seed, int32_t* out_tokens, int32_t* out_len,
                               float* step_logits_host, int32_t* n_steps);
 
+/* -------------------------------------------------------------- tokenizer */
+
+/* Host-side text <-> ids for the two ends of the token loop.  Runs on the CPU
+ * (as in grad.cpp); nothing here touches the GPU. */
+typedef struct gh_tokenizer gh_tokenizer;
+
+typedef struct gh_tokenizer_info {
+    uint32_t kind;        /* TokenizerKind, fingerprint.h:15-18: 2 = byte-level BPE */
+    int32_t vocab_size;   /* Tokenizer::vocab_size */
+    int32_t eos_id;       /* Tokenizer::eos_id ("<|endoftext|>"), -1 when absent */
+    int32_t n_merges;
+    int32_t n_specials;
+    uint64_t fingerprint; /* Tokenizer::fingerprint; what a checkpoint's TKFP trailer records */
+} gh_tokenizer_info;
+
+/* load_tokenizer (tokenizer.h:52, tokenizer.cpp:119-124): opens a "GTOK" v2 file
+ * (ByteBpe::load, byte_bpe.cpp:676-744) with the same validation and messages.
+ * A file that does not start with "GTOK" is a v1 cache in grad.cpp; those are
+ * refused here with GH_ERR_RUNTIME. */
+gh_status gh_tokenizer_load(const char* path, gh_tokenizer** out);
+/* ByteBpe(merges, specials) (byte_bpe.h:50-53): merges is n_merges x 2 ids;
+ * specials[i] has special_lens[i] bytes.  GH_ERR_INVALID_ARGUMENT with the
+ * constructor's messages. */
+gh_status gh_tokenizer_from_merges(const int32_t* merges, int32_t n_merges, const char* const* specials,
+                                   const int32_t* special_lens, int32_t n_specials, gh_tokenizer** out);
+/* Tokenizer::save (byte_bpe.cpp:655-674): writes a file grad.cpp loads. */
+gh_status gh_tokenizer_save(const gh_tokenizer* t, const char* path);
+void gh_tokenizer_free(gh_tokenizer* t);
+gh_status gh_tokenizer_get_info(const gh_tokenizer* t, gh_tokenizer_info* out);
+/* Tokenizer::special_id (tokenizer.h:33): *id = -1 when token is not special. */
+gh_status gh_tokenizer_special_id(const gh_tokenizer* t, const char* token, size_t len, int32_t* id);
+/* Tokenizer::encode (with_specials != 0) / ByteBpe::encode_ordinary (== 0),
+ * byte_bpe.cpp:555-591.  *n receives the number of ids of the whole text; at
+ * most cap of them are written to ids (call with cap = 0 to size a buffer). */
+gh_status gh_tokenizer_encode(const gh_tokenizer* t, const char* text, size_t len, int32_t with_specials,
+                              int32_t* ids, size_t cap, size_t* n);
+/* Tokenizer::decode (byte_bpe.cpp:649-653): bytes of the ids, concatenated;
+ * *len receives their total, at most cap are written (no terminator).
+ * GH_ERR_OUT_OF_RANGE for an id outside the vocabulary. */
+gh_status gh_tokenizer_decode(const gh_tokenizer* t, const int32_t* ids, size_t n, char* out, size_t cap,
+                              size_t* len);
+/* pretok::split (pretokenize.h:44, pretokenize.cpp:159-167): the end offset of
+ * every piece of text under GPT-2's pattern; *n receives the number of pieces,
+ * at most cap offsets are written. */
+gh_status gh_pretokenize(const char* text, size_t len, size_t* ends, size_t cap, size_t* n);
+/* pretok::classify (pretokenize.h:36): 0 other, 1 letter, 2 number, 3 white space. */
+int32_t gh_codepoint_class(uint32_t codepoint);
+
 /* ------------------------------------------------------------ measurement */
 
 /* GPU time of the last gh_session_generate call, from HIP events recorded on
