@@ -21,10 +21,22 @@ HIPCC_FLAGS = [
 SOURCES = ["engine.hip", "checkpoint.cpp", "tokenizer.cpp"]
 
 
+BIN_DIR = os.path.join(PKG, "bin")
+CLI = os.path.join(BIN_DIR, "gradhip-generate")
+INCLUDE = os.path.join(os.path.dirname(PKG), "include")
+
+
 def build(verbose: bool = True) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc, *HIPCC_FLAGS, "-o", LIB, *[os.path.join(CSRC, s) for s in SOURCES]]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    # the command-line caller: plain C++ over the header-only adapter
+    os.makedirs(BIN_DIR, exist_ok=True)
+    cmd = ["g++", "-std=c++20", "-O2", "-Wall", "-Wextra", "-I", INCLUDE, os.path.join(PKG, "cli", "generate.cpp"),
+           "-o", CLI, "-L", LIB_DIR, "-lgradhip", "-Wl,-rpath,$ORIGIN/../lib"]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

@@ -8,7 +8,9 @@
 //     grad::GPTModel::load            -> gradhip::GPTModel::load      (gpt_model.h:87)
 //     grad::InferenceSession          -> gradhip::InferenceSession    (inference.h:16-29)
 //     grad::TextGen                   -> gradhip::TextGen             (text_gen.h:12-38)
-//     grad::Tokenizer (decode only)   -> gradhip::Tokenizer           (tokenizer.h:20-43)
+//     grad::Tokenizer                 -> gradhip::Tokenizer           (tokenizer.h:20-43)
+//     grad::ByteBpe, load_tokenizer   -> gradhip::ByteBpe, gradhip::load_tokenizer
+//                                                                      (byte_bpe.h:37-113, tokenizer.h:52)
 //
 // The model lives on the GPU; there is no CPU path behind these classes.
 #pragma once
@@ -16,12 +18,15 @@
 #include "gradhip.h"
 
 #include <cstdint>
+#include <cstdio>
 #include <functional>
+#include <memory>
 #include <optional>
 #include <random>
 #include <span>
 #include <stdexcept>
 #include <string>
+#include <string_view>
 #include <utility>
 #include <vector>
 
@@ -47,12 +52,115 @@ struct TokenizerFingerprint {
     bool operator==(const TokenizerFingerprint&) const = default;
 };
 
-// The part of grad::Tokenizer the generation path uses (text_gen.cpp:122-125).
+// "v1" / "v2" and "v2:0123456789abcdef" (tokenizer.cpp:17-32).
+inline const char* tokenizer_kind_flag(TokenizerKind kind) {
+    return kind == TokenizerKind::BpeV1 ? "v1" : kind == TokenizerKind::ByteBpe ? "v2" : "unknown";
+}
+inline std::string to_string(const TokenizerFingerprint& f) {
+    char hex[17];
+    std::snprintf(hex, sizeof hex, "%016llx", static_cast<unsigned long long>(f.hash));
+    return std::string(tokenizer_kind_flag(f.kind)) + ":" + hex;
+}
+
+// grad::Tokenizer (tokenizer.h:20-43).  The generation path only calls decode
+// (text_gen.cpp:122-125), so a wrapper around another tokenizer need only
+// override that; the other members throw std::logic_error unless overridden.
 class Tokenizer {
 public:
     virtual ~Tokenizer() = default;
     [[nodiscard]] virtual std::string decode(std::span<const int> ids) const = 0;
+    [[nodiscard]] virtual std::vector<int> encode(std::string_view) const { unsupported("encode"); }
+    [[nodiscard]] virtual TokenizerKind kind() const { unsupported("kind"); }
+    [[nodiscard]] virtual int vocab_size() const { unsupported("vocab_size"); }
+    [[nodiscard]] virtual std::optional<int> eos_id() const { unsupported("eos_id"); }
+    [[nodiscard]] virtual std::optional<int> special_id(std::string_view) const { unsupported("special_id"); }
+    [[nodiscard]] virtual std::uint64_t fingerprint() const { unsupported("fingerprint"); }
+    [[nodiscard]] TokenizerFingerprint identity() const { return {kind(), fingerprint()}; }
+    virtual void save(const std::string&) const { unsupported("save"); }
+
+private:
+    [[noreturn]] static void unsupported(const char* what) {
+        throw std::logic_error(std::string("gradhip::Tokenizer::") + what + " is not implemented by this tokenizer");
+    }
 };
+
+// grad::ByteBpe (byte_bpe.h:37-113) without the trainer: the lossless byte-level
+// BPE of "GTOK" version 2 files.  Runs on the host.
+class ByteBpe final : public Tokenizer {
+public:
+    using Merge = std::pair<int, int>;
+    static constexpr std::string_view kEndOfText = "<|endoftext|>";
+
+    // Throws std::invalid_argument with the reference constructor's messages.
+    explicit ByteBpe(const std::vector<Merge>& merges,
+                     const std::vector<std::string>& specials = {std::string(kEndOfText)}) {
+        std::vector<int32_t> flat;
+        for (const Merge& m : merges) {
+            flat.push_back(m.first);
+            flat.push_back(m.second);
+        }
+        std::vector<const char*> ptrs;
+        std::vector<int32_t> lens;
+        for (const std::string& sp : specials) {
+            ptrs.push_back(sp.data());
+            lens.push_back(static_cast<int32_t>(sp.size()));
+        }
+        check(gh_tokenizer_from_merges(flat.data(), static_cast<int32_t>(merges.size()), ptrs.data(), lens.data(),
+                                       static_cast<int32_t>(specials.size()), &t_));
+        check(gh_tokenizer_get_info(t_, &info_));
+    }
+    // Throws std::runtime_error("Tokenizer file <path>: ...") like ByteBpe::load (byte_bpe.cpp:676-744).
+    [[nodiscard]] static ByteBpe load(const std::string& path) {
+        gh_tokenizer* t = nullptr;
+        check(gh_tokenizer_load(path.c_str(), &t));
+        return ByteBpe(t);
+    }
+    ByteBpe(const ByteBpe&) = delete;
+    ByteBpe& operator=(const ByteBpe&) = delete;
+    ByteBpe(ByteBpe&& o) noexcept : t_(std::exchange(o.t_, nullptr)), info_(o.info_) {}
+    ~ByteBpe() override { gh_tokenizer_free(t_); }
+
+    [[nodiscard]] TokenizerKind kind() const override { return TokenizerKind::ByteBpe; }
+    [[nodiscard]] std::vector<int> encode(std::string_view text) const override { return run_encode(text, 1); }
+    [[nodiscard]] std::vector<int> encode_ordinary(std::string_view text) const { return run_encode(text, 0); }
+    // Throws std::out_of_range for an id outside the vocabulary.
+    [[nodiscard]] std::string decode(std::span<const int> ids) const override {
+        std::size_t len = 0;
+        check(gh_tokenizer_decode(t_, ids.data(), ids.size(), nullptr, 0, &len));
+        std::string out(len, '\0');
+        check(gh_tokenizer_decode(t_, ids.data(), ids.size(), out.data(), out.size(), &len));
+        return out;
+    }
+    [[nodiscard]] int vocab_size() const override { return info_.vocab_size; }
+    [[nodiscard]] std::optional<int> eos_id() const override {
+        return info_.eos_id < 0 ? std::nullopt : std::optional<int>(info_.eos_id);
+    }
+    [[nodiscard]] std::optional<int> special_id(std::string_view token) const override {
+        int32_t id = -1;
+        check(gh_tokenizer_special_id(t_, token.data(), token.size(), &id));
+        return id < 0 ? std::nullopt : std::optional<int>(id);
+    }
+    [[nodiscard]] std::uint64_t fingerprint() const override { return info_.fingerprint; }
+    void save(const std::string& path) const override { check(gh_tokenizer_save(t_, path.c_str())); }
+
+private:
+    explicit ByteBpe(gh_tokenizer* t) : t_(t) { check(gh_tokenizer_get_info(t_, &info_)); }
+    std::vector<int> run_encode(std::string_view text, int32_t with_specials) const {
+        std::vector<int> ids(text.size());  // never more ids than bytes
+        std::size_t n = 0;
+        check(gh_tokenizer_encode(t_, text.data(), text.size(), with_specials, ids.data(), ids.size(), &n));
+        ids.resize(n);
+        return ids;
+    }
+    gh_tokenizer* t_ = nullptr;
+    gh_tokenizer_info info_{};
+};
+
+// load_tokenizer (tokenizer.h:52).  grad.cpp also opens v1 caches here; this
+// library reads "GTOK" files only and throws std::runtime_error for anything else.
+[[nodiscard]] inline std::unique_ptr<Tokenizer> load_tokenizer(const std::string& path) {
+    return std::make_unique<ByteBpe>(ByteBpe::load(path));
+}
 
 class GPTModel {
 public:
@@ -106,6 +214,28 @@ private:
     gh_model* m_ = nullptr;
     gh_config cfg_{};
 };
+
+// The CLI's guard before generating (src/cli/common.cpp:254-268): a checkpoint
+// that records a tokenizer fingerprint is only used with that tokenizer.  Returns
+// false (after a warning on stderr) when the checkpoint records none; throws
+// std::runtime_error with the reference's message on a mismatch.
+inline bool check_tokenizer_matches(const GPTModel& model, const Tokenizer& tokenizer,
+                                    const std::string& checkpoint_path) {
+    const std::optional<TokenizerFingerprint> recorded = model.getTokenizerFingerprint();
+    if (!recorded) {
+        std::fprintf(stderr,
+                     "Warning: %s records no tokenizer fingerprint (it predates tokenizer v2); using the %s "
+                     "tokenizer unverified\n",
+                     checkpoint_path.c_str(), tokenizer_kind_flag(tokenizer.kind()));
+        return false;
+    }
+    if (!(*recorded == tokenizer.identity())) {
+        throw std::runtime_error("tokenizer " + to_string(tokenizer.identity()) + " is not the one "
+                                 + checkpoint_path + " was trained with (" + to_string(*recorded)
+                                 + "); its token ids would mean different text");
+    }
+    return true;
+}
 
 // Incremental decoding with a KV cache (inference.h:16-29).  The model must
 // outlive the session; the pointer step() returns is valid until the next step().

@@ -1,0 +1,75 @@
+"""Text in, text out: gradhip-generate (the `grad generate`-shaped caller, grad.cpp
+src/cli/generate.cpp:61-107) encodes a prompt with a GTOK file, runs both loops on the
+GPU and prints decoded text.  Checked against the CPU restatements of the tokenizer and
+of the token loop; the tokenizer fingerprint guard against src/cli/common.cpp:254-268."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+import oracle_lib as O
+from gradhip import synth
+from helpers import lively_std
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+import tokenizer_ref as R  # noqa: E402
+
+CLI = os.path.join(ROOT, "grad.cpp_amd", "bin", "gradhip-generate")
+TEXT = "Once upon a time, the little cat said: don't go!\nThe end. "
+
+
+@pytest.fixture(scope="module")
+def setup(tmp_path_factory):
+    d = tmp_path_factory.mktemp("cli")
+    tok = R.train((TEXT * 3 + "the cat sat on the mat and the cat ran to the hat\n" * 5).encode(), 330)
+    (d / "t.tok").write_bytes(tok.file_image())
+    cfg = synth.Config(synth.ARCH_MODERN, tok.vocab_size, 128, 2, 2, 64)
+    W = synth.make_weights(cfg, 31, std=lively_std(cfg), norm_noise=0.1)
+    synth.write_checkpoint(str(d / "m.bin"), cfg, W, fingerprint=(2, tok.fingerprint()))
+    synth.write_checkpoint(str(d / "other.bin"), cfg, W, fingerprint=(2, tok.fingerprint() ^ 1))
+    synth.write_checkpoint(str(d / "plain.bin"), cfg, W)
+    return d, tok, cfg, O.Model.from_tensors(cfg, W)
+
+
+def run(*args):
+    assert os.path.exists(CLI), "gradhip-generate is not built; run __graft_entry__.build()"
+    return subprocess.run([CLI, *[str(a) for a in args]], capture_output=True, timeout=120)
+
+
+def test_generate_prints_the_oracles_text(setup):
+    d, tok, cfg, om = setup
+    prompt = "the little cat"
+    out = run(d / "m.bin", d / "t.tok", prompt, "--max-tokens", 12, "--temperature", 0.8, "--top-k", 5, "--top-p",
+              0.9, "--repetition-penalty", 1.1, "--seed", 77)
+    assert out.returncode == 0, out.stdout + out.stderr
+    ids = tok.encode(prompt.encode())
+    greedy = O.generate_greedy(om, ids, 12, 1.1)
+    sampled = O.generate_sample(om, ids, synth.uniforms(12, 77), 0.8, 12, 1.1, 5, 0.9)
+    want = (b"\ngradhip Generation\n\n"
+            + f"Tokenizer: {d / 't.tok'} (v2, vocab {tok.vocab_size})\n".encode()
+            + b"\n--- Greedy Decoding ---\n\n" + f'Prompt: "{prompt}"\n'.encode() + tok.decode(greedy) + b"\n"
+            + b"\n--- Sampling (temp=0.8, top-k=5, top-p=0.9) ---\n\n" + f'Prompt: "{prompt}"\n'.encode()
+            + tok.decode(sampled) + b"\n")
+    assert out.stdout == want
+    only = run(d / "m.bin", d / "t.tok", prompt, "--max-tokens", 12, "--repetition-penalty", 1.1, "--greedy")
+    assert only.returncode == 0 and b"Sampling" not in only.stdout and tok.decode(greedy) in only.stdout
+
+
+def test_fingerprint_guard_and_exit_codes(setup):
+    d, tok, cfg, om = setup
+    out = run(d / "other.bin", d / "t.tok", "the cat")
+    assert out.returncode == 1
+    fp = tok.fingerprint()
+    assert (f"Error: tokenizer v2:{fp:016x} is not the one {d / 'other.bin'} was trained with "
+            f"(v2:{fp ^ 1:016x}); its token ids would mean different text").encode() in out.stderr
+    out = run(d / "plain.bin", d / "t.tok", "the cat", "--max-tokens", 3, "--greedy")
+    assert out.returncode == 0
+    assert b"records no tokenizer fingerprint (it predates tokenizer v2); using the v2 tokenizer unverified" in out.stderr
+    assert run(d / "m.bin", d / "t.tok").returncode == 2            # usage
+    assert run(d / "m.bin", d / "t.tok", "x", "--top-p", 2).returncode == 2
+    out = run(d / "missing.bin", d / "t.tok", "x")
+    assert out.returncode == 1 and b"Could not open checkpoint for reading" in out.stderr
