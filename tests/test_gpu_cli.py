@@ -73,3 +73,29 @@ def test_fingerprint_guard_and_exit_codes(setup):
     assert run(d / "m.bin", d / "t.tok", "x", "--top-p", 2).returncode == 2
     out = run(d / "missing.bin", d / "t.tok", "x")
     assert out.returncode == 1 and b"Could not open checkpoint for reading" in out.stderr
+
+
+def test_bench_writes_the_reference_schema(tmp_path):
+    """gradhip-bench: grad bench's generation section (src/cli/bench.cpp:269-286) and its JSON
+    schema (:112-172)."""
+    import json
+    exe = os.path.join(ROOT, "grad.cpp_amd", "bin", "gradhip-bench")
+    assert os.path.exists(exe), "gradhip-bench is not built; run __graft_entry__.build()"
+    path = tmp_path / "bench.json"
+    out = subprocess.run([exe, "--trials", "3", "--json", str(path)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "Generation throughput" in out.stdout and "median:" in out.stdout
+    j = json.loads(path.read_text())
+    assert list(j) == ["schema_version", "timestamp_utc", "engine", "version", "git_sha", "build_type", "compiler",
+                       "system", "metal_available", "metal_fp16", "device", "parameters", "config", "protocol",
+                       "training_steps_per_second", "training_tokens_per_second", "generation_tokens_per_second",
+                       "median_training_steps_per_second", "median_training_tokens_per_second",
+                       "median_generation_tokens_per_second", "peak_rss_mb", "metal_stream_per_step",
+                       "metal_peak_live_mb"]
+    assert j["schema_version"] == 1 and j["config"]["vocab"] == 5000 and j["config"]["d_model"] == 512
+    # E, P, 6 x (4 d^2 + 4 d + 8 d^2 + 5 d + 4 d) and the final norm: the 22M configuration
+    assert j["parameters"] == 5000 * 512 + 1024 * 512 + 6 * (12 * 512 * 512 + 13 * 512) + 2 * 512
+    rates = j["generation_tokens_per_second"]
+    assert len(rates) == 3 and all(r > 0 for r in rates)
+    assert abs(j["median_generation_tokens_per_second"] - sorted(rates)[1]) < 1e-3
+    assert subprocess.run([exe, "--trials", "0"], capture_output=True).returncode == 2
