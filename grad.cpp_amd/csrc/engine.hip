@@ -365,6 +365,8 @@ struct Session {
     // prompt pass (all prompt tokens at once): row-major [rows][width] activations
     float *pp_x = nullptr, *pp_q = nullptr, *pp_attn = nullptr, *pp_norm = nullptr, *pp_hidden = nullptr;
     size_t pp_rows = 0;
+    float* score_logits = nullptr;  // [score_rows][vocab] logits of a block of rows being scored
+    size_t score_rows = 0;
 
     // persistent engine
     Cell* cells = nullptr;  // xa, xb, q, kn, vn, at (d each), hid (F), token (1)
@@ -414,7 +416,7 @@ struct Session {
                         static_cast<void*>(logit_log), static_cast<void*>(cells),
                         static_cast<void*>(ctl), static_cast<void*>(pp_x), static_cast<void*>(pp_q),
                         static_cast<void*>(pp_attn), static_cast<void*>(pp_norm),
-                        static_cast<void*>(pp_hidden)})
+                        static_cast<void*>(pp_hidden), static_cast<void*>(score_logits)})
             if (p) (void)hipFree(p);
         if (host_logits) (void)hipHostFree(host_logits);
         if (host_ids) (void)hipHostFree(host_ids);
@@ -1046,9 +1048,52 @@ static void project_rows(Session& s, GemvParams g, int M) {
     HIP_CHECK(hipGetLastError());
 }
 
+// Where a scored pass leaves its result: targets and nll are device arrays
+// [batch][len] indexed like the ids of the pass.
+struct ScoreSink {
+    const int* targets;
+    float* nll;
+};
+
+// Final norm, logits and the target's negative log-likelihood for rows
+// pp_x[0 .. M) of a slice (row m = seq * n + t, position t0 + t), a block of rows
+// at a time so that the logits of a block stay a modest buffer.
+static void score_rows(Session& s, const ScoreSink& sink, int M, int n, int t0, int len) {
+    const Model& m = *s.m;
+    const Shape& sh = m.shape;
+    const size_t V = sh.vocab;
+    const size_t want = std::min<size_t>(static_cast<size_t>(M),
+                                         std::max<size_t>(128, ((size_t{64} << 20) / V) / 128 * 128));
+    if (s.score_rows < want) {
+        if (s.score_logits) HIP_CHECK(hipFree(s.score_logits));
+        s.score_logits = nullptr;
+        dev_alloc(s.score_logits, want * V);
+        s.score_rows = want;
+    }
+    for (int r0 = 0; r0 < M; r0 += static_cast<int>(s.score_rows)) {
+        const int rows = std::min<int>(static_cast<int>(s.score_rows), M - r0);
+        GemvParams g{};
+        g.W = m.E;
+        g.N = sh.vocab;
+        g.K = sh.d_model;
+        g.in = s.pp_x + static_cast<size_t>(r0) * sh.d_model;
+        g.in_stride = sh.d_model;
+        g.gamma = m.gf;
+        g.beta = m.bf;
+        g.out = s.score_logits;
+        g.out_stride = sh.vocab;
+        if (sh.modern()) project_rows<PRO_RMSNORM, EPI_STORE>(s, g, rows);
+        else project_rows<PRO_LAYERNORM, EPI_STORE>(s, g, rows);
+        hipLaunchKernelGGL(nll_rows_kernel, dim3(rows), dim3(256), 0, s.stream, s.score_logits, sh.vocab, r0, n, t0,
+                           len, sink.targets, sink.nll);
+        HIP_CHECK(hipGetLastError());
+    }
+}
+
 // Tokens hist[n_hist .. n_hist + len) of every sequence, positions pos .. pos + len.
-// Equivalent to len step() calls (text_gen.cpp:44-46); only the last logits are formed.
-static void prompt_pass(Session& s, int len) {
+// Equivalent to len step() calls (text_gen.cpp:44-46); only the last logits are
+// formed unless a sink asks for the likelihood of a target at every position.
+static void prompt_pass(Session& s, int len, const ScoreSink* sink = nullptr) {
     const Model& m = *s.m;
     const Shape& sh = m.shape;
     const int d = sh.d_model, F = sh.d_ff(), B = s.B;
@@ -1149,6 +1194,7 @@ static void prompt_pass(Session& s, int len) {
             g.out_stride = d;
             project_rows<PRO_PLAIN, EPI_RESID>(s, g, M);
         }
+        if (sink) score_rows(s, *sink, M, n, t0, len);
         if (t0 + n == len) {
             hipLaunchKernelGGL(take_last_rows_kernel, dim3((d + 255) / 256, B), dim3(256), 0, st, s.pp_x, n,
                                s.x, d);
@@ -1573,6 +1619,65 @@ gh_status gh_session_prefill(gh_session* sess, const int32_t* ids, int32_t len,
         HIP_CHECK(hipStreamSynchronize(s.stream));
         check_persist_abort(s);
         if (last_logits_host) std::memcpy(last_logits_host, s.host_logits, s.B * V * sizeof(float));
+    });
+}
+
+gh_status gh_session_score(gh_session* sess, const int32_t* ids, const int32_t* targets, int32_t len,
+                           float* nll_host) {
+    return guard([&] {
+        if (!sess || !ids || !targets || !nll_host) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        if (len < 0) throw ApiError{GH_ERR_INVALID_ARGUMENT, "negative length"};
+        if (len == 0) return;
+        if (s.pos + len > s.m->shape.max_len)
+            throw ApiError{GH_ERR_RUNTIME, "InferenceSession: context exceeds max_len"};
+        const size_t n = static_cast<size_t>(s.B) * len;
+        check_ids(s, ids, n);
+        check_ids(s, targets, n);
+        const int base = s.n_hist;
+        for (int b = 0; b < s.B; b++) {
+            std::memcpy(s.host_ids + static_cast<size_t>(b) * s.hist_stride,
+                        ids + static_cast<size_t>(b) * len, len * sizeof(int));
+            HIP_CHECK(hipMemcpyAsync(s.hist + static_cast<size_t>(b) * s.hist_stride + base,
+                                     s.host_ids + static_cast<size_t>(b) * s.hist_stride,
+                                     len * sizeof(int), hipMemcpyHostToDevice, s.stream));
+        }
+        // targets and results live for this call only
+        struct Scratch {
+            int* targets = nullptr;
+            float* nll = nullptr;
+            ~Scratch() {
+                if (targets) (void)hipFree(targets);
+                if (nll) (void)hipFree(nll);
+            }
+        } tmp;
+        dev_alloc(tmp.targets, n);
+        dev_alloc(tmp.nll, n);
+        HIP_CHECK(hipMemcpyAsync(tmp.targets, targets, n * sizeof(int), hipMemcpyHostToDevice, s.stream));
+        const ScoreSink sink{tmp.targets, tmp.nll};
+        if (s.use_prompt_pass && prompt_pass_ok(s, len)) {
+            prompt_pass(s, len, &sink);
+        } else {
+            // token by token: every step leaves the logits of its position
+            const int V = s.m->shape.vocab;
+            for (int t = 0; t < len; t++) {
+                if (s.engine == GH_ENGINE_PERSISTENT) {
+                    persist_run(s, 1, 1, 0, false, nullptr, nullptr, 0, 0, nullptr);  // token from the history
+                } else {
+                    hipLaunchKernelGGL(load_tok_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
+                                       s.hist_stride, base + t, s.tok, s.B);
+                    HIP_CHECK(hipGetLastError());
+                    run_step(s);
+                }
+                hipLaunchKernelGGL(nll_rows_kernel, dim3(s.B), dim3(256), 0, s.stream, s.logits, V, 0, 1, t, len,
+                                   sink.targets, sink.nll);
+                HIP_CHECK(hipGetLastError());
+            }
+            if (s.engine != GH_ENGINE_PERSISTENT) s.n_hist += len;
+        }
+        HIP_CHECK(hipMemcpyAsync(nll_host, tmp.nll, n * sizeof(float), hipMemcpyDeviceToHost, s.stream));
+        HIP_CHECK(hipStreamSynchronize(s.stream));
+        check_persist_abort(s);
     });
 }
 

@@ -252,4 +252,28 @@ __global__ void take_last_rows_kernel(const float* __restrict__ x, int len, floa
 // pos_++ at the end of a step (inference.cpp:256).
 __global__ void advance_kernel(DevState* st) { st->pos += 1; }
 
+// Negative log-likelihood of one target per logits row: Variable::cross_entropy's
+// log_softmax + nll_loss (variable.cpp:589-592) before the mean over rows.  One
+// workgroup per row; row r of this launch is row `row0 + r` of a prompt pass
+// whose row m = seq * slice_len + t holds position t0 + t of sequence seq.
+// nll[seq * len + t0 + t] = log(sum_j exp(x_j - max)) + max - x_target.
+__global__ __launch_bounds__(256) void nll_rows_kernel(const float* __restrict__ logits, int V, int row0,
+                                                       int slice_len, int t0, int len,
+                                                       const int* __restrict__ targets, float* __restrict__ nll) {
+    __shared__ float scratch[4];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* x = logits + static_cast<size_t>(r) * V;
+    float mx = -INFINITY;
+    for (int j = tid; j < V; j += 256) mx = fmaxf(mx, x[j]);
+    mx = block_max(mx, scratch);
+    float sum = 0.0f;
+    for (int j = tid; j < V; j += 256) sum += expf(x[j] - mx);
+    sum = block_sum(sum, scratch);
+    if (tid == 0) {
+        const int m = row0 + r, seq = m / slice_len, t = m - seq * slice_len;
+        const size_t at = static_cast<size_t>(seq) * len + t0 + t;
+        nll[at] = (logf(sum) + mx) - x[targets[at]];
+    }
+}
+
 }  // namespace gh

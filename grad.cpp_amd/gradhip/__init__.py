@@ -74,6 +74,7 @@ SYMBOLS = {
     "gh_session_step": (C.c_int, [_vp, _i32p, _f32p]),
     "gh_session_logits": (C.c_int, [_vp, C.POINTER(_f32p)]),
     "gh_session_prefill": (C.c_int, [_vp, _i32p, C.c_int32, _f32p]),
+    "gh_session_score": (C.c_int, [_vp, _i32p, _i32p, C.c_int32, _f32p]),
     "gh_session_position": (C.c_int32, [_vp]),
     "gh_session_capacity": (C.c_int32, [_vp]),
     "gh_session_vocab": (C.c_int32, [_vp]),
@@ -334,6 +335,16 @@ class Session:
         out = np.empty((self.batch, self.vocab), dtype=np.float32)
         _check(load_library().gh_session_prefill(self._h, ids.ctypes.data_as(_i32p), ids.shape[1],
                                                  out.ctypes.data_as(_f32p)))
+        return out
+
+    def score(self, ids, targets) -> np.ndarray:
+        """Negative log-likelihood of targets[b, t] at every position (what `grad eval` averages)."""
+        ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(self.batch, -1)
+        targets = np.ascontiguousarray(targets, dtype=np.int32).reshape(self.batch, -1)
+        assert ids.shape == targets.shape
+        out = np.empty(ids.shape, dtype=np.float32)
+        _check(load_library().gh_session_score(self._h, ids.ctypes.data_as(_i32p), targets.ctypes.data_as(_i32p),
+                                               ids.shape[1], out.ctypes.data_as(_f32p)))
         return out
 
     def read_kv(self, seq, layer, kv, pos) -> np.ndarray:

@@ -245,6 +245,18 @@ gh_status gh_pretokenize(const char* text, size_t len, size_t* ends, size_t cap,
 /* pretok::classify (pretokenize.h:36): 0 other, 1 letter, 2 number, 3 white space. */
 int32_t gh_codepoint_class(uint32_t codepoint);
 
+/* ------------------------------------------------------------------ scoring */
+
+/* What `grad eval` computes per window (training::mean_loss, src/training/trainer.cpp:319-340:
+ * GPTModel::forward, gpt_model.cpp:74-142, then Variable::cross_entropy,
+ * variable.cpp:589-592), before the mean: nll_host[b * len + t] = -log
+ * softmax(logits at position t of sequence b)[targets[b * len + t]], all
+ * positions in one pass over the weights.  ids and targets are batch x len.
+ * The pass fills the KV cache and advances the position like gh_session_prefill
+ * (call gh_session_reset between windows); same errors as gh_session_prefill. */
+gh_status gh_session_score(gh_session* s, const int32_t* ids, const int32_t* targets, int32_t len,
+                           float* nll_host);
+
 /* ------------------------------------------------------------ measurement */
 
 /* GPU time of the last gh_session_generate call, from HIP events recorded on

@@ -260,6 +260,16 @@ public:
         return logits;
     }
 
+    // Negative log-likelihood of targets[t] at every position of ids, all positions
+    // in one pass (what training::mean_loss averages, src/training/trainer.cpp:319-340).
+    // Continues from the current position and fills the cache like step() would.
+    [[nodiscard]] std::vector<float> score(const std::vector<int>& ids, const std::vector<int>& targets) {
+        if (ids.size() != targets.size()) throw std::invalid_argument("score: ids and targets differ in length");
+        std::vector<float> nll(ids.size());
+        check(gh_session_score(s_, ids.data(), targets.data(), static_cast<int32_t>(ids.size()), nll.data()));
+        return nll;
+    }
+
     int position() const { return gh_session_position(s_); }
     int capacity() const { return gh_session_capacity(s_); }
     int vocabSize() const { return gh_session_vocab(s_); }

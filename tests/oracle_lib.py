@@ -225,3 +225,21 @@ def generate_sample(model, prompt, uniforms, temperature=1.0, max_tokens=50, pen
                                   _fp(sl) if want_logits else None, C.byref(ns)))
     toks = out[:n.value].copy()
     return (toks, sl[:ns.value]) if want_logits else toks
+
+
+def nll_rows(logits, targets):
+    """Negative log-likelihood of targets[i] under softmax(logits[i]), in float64:
+    Variable::cross_entropy's log_softmax + nll_loss (variable.cpp:589-592) before the mean
+    over rows.  Pinned by closed forms in tests/test_oracle_textgen.py."""
+    x = np.asarray(logits, dtype=np.float64)
+    m = x.max(axis=-1, keepdims=True)
+    lse = np.log(np.exp(x - m).sum(axis=-1)) + m[..., 0]
+    return lse - np.take_along_axis(x, np.asarray(targets)[..., None], axis=-1)[..., 0]
+
+
+def score(model, ids, targets):
+    """Per-position NLL of one sequence, logits from step() (what `grad eval` averages,
+    training/trainer.cpp:319-340, with the full-sequence forward replaced by the token loop,
+    which the reference's own parity tests tie together, sanity_tests.cpp:293-333)."""
+    s = Session(model)
+    return np.array([nll_rows(s.step(int(t)), int(g)) for t, g in zip(ids, targets)])

@@ -215,3 +215,24 @@ def test_sample_loop_consumes_one_uniform_per_token():
     a = O.generate_sample(om, [1, 2, 3], synth.uniforms(8, 1), 1.0, 8, 1.0, 1, 1.0)
     b = O.generate_sample(om, [1, 2, 3], synth.uniforms(8, 2), 1.0, 8, 1.0, 1, 1.0)
     assert a.tolist() == b.tolist() == O.generate_greedy(om, [1, 2, 3], 8, 1.0).tolist()
+
+
+def test_nll_rows_closed_forms():
+    """The scoring restatement against what the mathematics fixes."""
+    V = 37
+    rng = np.random.default_rng(3)
+    # uniform logits: -log(1/V) whatever the target and the level
+    assert np.allclose(O.nll_rows(np.full((4, V), 2.5), [0, 5, 36, 7]), np.log(V), atol=1e-12)
+    # two classes: softplus of the logit difference
+    d = rng.normal(size=6) * 3
+    x = np.stack([np.zeros(6), d], axis=1)
+    assert np.allclose(O.nll_rows(x, np.zeros(6, int)), np.log1p(np.exp(d)), atol=1e-12)
+    assert np.allclose(O.nll_rows(x, np.ones(6, int)), np.log1p(np.exp(-d)), atol=1e-12)
+    # shift invariance and the definition through probabilities
+    x = rng.normal(size=(5, V)) * 4
+    t = rng.integers(0, V, 5)
+    assert np.allclose(O.nll_rows(x + 100.0, t), O.nll_rows(x, t), atol=1e-9)
+    p = np.exp(x) / np.exp(x).sum(axis=1, keepdims=True)
+    assert np.allclose(O.nll_rows(x, t), -np.log(p[np.arange(5), t]), atol=1e-12)
+    # probabilities sum to one: exp(-nll) over all targets
+    assert np.allclose(sum(np.exp(-O.nll_rows(x, np.full(5, j))) for j in range(V)), 1.0, atol=1e-12)
