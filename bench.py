@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # (32-token prompt already cached): FETCH_SIZE and WRITE_SIZE, converted to bytes
 # with the factors a 1 GiB copy kernel gives for the same counters.
 PMC_STEPS_PER_LAUNCH = 224
-PMC_FETCH_BYTES_PER_LAUNCH = 31_344_096 * 2048  # counter reads 1 per 2 KiB fetched
-PMC_WRITE_BYTES_PER_LAUNCH = 540_302 * 1024     # counter reads 1 per KiB written
+PMC_FETCH_BYTES_PER_LAUNCH = 31_344_952 * 2048  # counter reads 1 per 2 KiB fetched
+PMC_WRITE_BYTES_PER_LAUNCH = 541_326 * 1024     # counter reads 1 per KiB written
 
 
 def step_bytes(cfg, batch, ctx):

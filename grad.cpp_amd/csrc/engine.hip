@@ -515,7 +515,8 @@ static int project(Session& s, GemvParams g, hipStream_t st) {
 }
 
 // final norm -> logits = h @ E^T (inference.cpp:251-254) from the rows in s.x
-static int enqueue_logits(Session& s) {
+// advance: the launch also ends the step (pos_++).
+static int enqueue_logits(Session& s, bool advance) {
     const Model& m = *s.m;
     const Shape& sh = m.shape;
     const bool modern = sh.modern();
@@ -530,6 +531,7 @@ static int enqueue_logits(Session& s) {
     g.beta = m.bf;
     g.out = s.logits;
     g.out_stride = sh.vocab;
+    g.advance = advance ? s.st : nullptr;
     return modern ? project<PRO_RMSNORM, EPI_STORE>(s, g, s.stream)
                   : project<PRO_LAYERNORM, EPI_STORE>(s, g, s.stream);
 }
@@ -629,11 +631,7 @@ static int enqueue_step(Session& s) {
         launches += project<PRO_PLAIN, EPI_RESID>(s, g, st);
     }
 
-    launches += enqueue_logits(s);
-
-    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, st, s.st);
-    HIP_CHECK(hipGetLastError());
-    launches++;
+    launches += enqueue_logits(s, /*advance=*/true);
     return launches;
 }
 
@@ -1206,7 +1204,7 @@ static void prompt_pass(Session& s, int len, const ScoreSink* sink = nullptr) {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, st, s.st, s.pos, s.n_hist, s.picks);
     HIP_CHECK(hipGetLastError());
     // logits of the last position, through the decode-size projection
-    enqueue_logits(s);
+    enqueue_logits(s, /*advance=*/false);
 }
 
 // Steps through `len` tokens already staged in the history at n_hist.. (the

@@ -33,6 +33,9 @@ struct GemvParams {
     const float* rope_cos;  // [max_len][head_size/2]
     const float* rope_sin;
     const DevState* st;
+    // EPI_STORE only: when set, the thread that stores element (0, 0) also ends the
+    // step, pos_++ (inference.cpp:256).  Nothing else in that launch reads the state.
+    DevState* advance;
     // Rows of one prompt pass: row m is token m % rows_per_seq of sequence
     // m / rows_per_seq and sits at position pos_base + m % rows_per_seq.
     // rows_per_seq == 0: one row per sequence, all at st->pos (a decode step).
@@ -61,6 +64,7 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, int b, int ro
         float* o = p.out + static_cast<size_t>(b) * p.out_stride;
         o[row] = v0 + (p.bias ? p.bias[row] : 0.0f);
         if (has1) o[row + 1] = v1 + (p.bias ? p.bias[row + 1] : 0.0f);
+        if (p.advance && b == 0 && row == 0) p.advance->pos += 1;
     } else if constexpr (EPI == EPI_RESID) {
         // y += b, then y += x @ W (inference.cpp:22-28)
         float* o = p.out + static_cast<size_t>(b) * p.out_stride;
@@ -249,8 +253,6 @@ __global__ void take_last_rows_kernel(const float* __restrict__ x, int len, floa
     if (j < d) rows[static_cast<size_t>(b) * d + j] = x[(static_cast<size_t>(b) * len + len - 1) * d + j];
 }
 
-// pos_++ at the end of a step (inference.cpp:256).
-__global__ void advance_kernel(DevState* st) { st->pos += 1; }
 
 // Negative log-likelihood of one target per logits row: Variable::cross_entropy's
 // log_softmax + nll_loss (variable.cpp:589-592) before the mean over rows.  One
