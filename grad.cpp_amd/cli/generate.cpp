@@ -11,8 +11,8 @@
 // guard is the same: a checkpoint that records a tokenizer is only used with it.
 // Exit codes follow src/cli/main.cpp:94-103: 2 for a usage error, 1 for any failure.
 #include "gradhip.hpp"
+#include "options.h"
 
-#include <cstdlib>
 #include <iostream>
 #include <sstream>
 #include <string>
@@ -20,69 +20,8 @@
 
 namespace {
 
-struct Usage : std::runtime_error {
-    using std::runtime_error::runtime_error;
-};
-
-struct Options {
-    std::string checkpoint, tokenizer, prompt;
-    int max_tokens = 150;  // generate.cpp:67
-    float temperature = 0.8f;
-    int top_k = 0;
-    float top_p = 1.0f;
-    float repetition_penalty = 1.2f;
-    bool greedy = false;
-    std::optional<std::uint64_t> seed;
-};
-
-template <class T>
-T number(const std::string& flag, const std::string& text) {
-    std::istringstream in(text);
-    T v{};
-    if (!(in >> v) || !in.eof()) throw Usage(flag + ": expected a number, got '" + text + "'");
-    return v;
-}
-
-Options parse(int argc, char** argv) {
-    Options o;
-    std::vector<std::string> positional;
-    for (int i = 1; i < argc; i++) {
-        const std::string a = argv[i];
-        const auto value = [&]() -> std::string {
-            if (i + 1 >= argc) throw Usage(a + ": missing value");
-            return argv[++i];
-        };
-        if (a == "--max-tokens") {
-            o.max_tokens = number<int>(a, value());
-            if (o.max_tokens < 1) throw Usage("--max-tokens: must be at least 1");
-        } else if (a == "--temperature") {
-            o.temperature = number<float>(a, value());
-            if (!(o.temperature > 0.0f)) throw Usage("--temperature: must be positive");
-        } else if (a == "--top-k") {
-            o.top_k = number<int>(a, value());
-            if (o.top_k < 0) throw Usage("--top-k: must be at least 0");
-        } else if (a == "--top-p") {
-            o.top_p = number<float>(a, value());
-            if (!(o.top_p > 0.0f) || o.top_p > 1.0f) throw Usage("--top-p: must be positive and at most 1");
-        } else if (a == "--repetition-penalty") {
-            o.repetition_penalty = number<float>(a, value());
-            if (!(o.repetition_penalty > 0.0f)) throw Usage("--repetition-penalty: must be positive");
-        } else if (a == "--greedy") {
-            o.greedy = true;
-        } else if (a == "--seed") {
-            o.seed = number<std::uint64_t>(a, value());
-        } else if (a.rfind("--", 0) == 0) {
-            throw Usage("unknown option " + a);
-        } else {
-            positional.push_back(a);
-        }
-    }
-    if (positional.size() != 3) throw Usage("usage: gradhip-generate <checkpoint> <tokenizer.tok> <prompt> [options]");
-    o.checkpoint = positional[0];
-    o.tokenizer = positional[1];
-    o.prompt = positional[2];
-    return o;
-}
+using gradhip::cli::Options;
+using gradhip::cli::Usage;
 
 // "temp=0.8", plus any cut that is on (generate.cpp:50-57).
 std::string describe(const Options& o) {
@@ -97,31 +36,34 @@ std::string describe(const Options& o) {
 
 int main(int argc, char** argv) {
     try {
-        const Options o = parse(argc, argv);
+        const Options o = gradhip::cli::parse(argc, argv, Options{});
+        if (o.positional.size() != 3)
+            throw Usage("usage: gradhip-generate <checkpoint> <tokenizer.tok> <prompt> [options]");
+        const std::string &checkpoint = o.positional[0], &tokenizer_path = o.positional[1], &text = o.positional[2];
         std::cout << "\ngradhip Generation\n" << std::endl;
-        const gradhip::GPTModel model = gradhip::GPTModel::load(o.checkpoint);
-        const std::unique_ptr<gradhip::Tokenizer> tokenizer = gradhip::load_tokenizer(o.tokenizer);
-        std::cout << "Tokenizer: " << o.tokenizer << " (" << gradhip::tokenizer_kind_flag(tokenizer->kind())
+        const gradhip::GPTModel model = gradhip::GPTModel::load(checkpoint);
+        const std::unique_ptr<gradhip::Tokenizer> tokenizer = gradhip::load_tokenizer(tokenizer_path);
+        std::cout << "Tokenizer: " << tokenizer_path << " (" << gradhip::tokenizer_kind_flag(tokenizer->kind())
                   << ", vocab " << tokenizer->vocab_size() << ")" << std::endl;
         if (tokenizer->vocab_size() != model.getVocabSize()) {
             throw std::runtime_error("tokenizer vocab " + std::to_string(tokenizer->vocab_size())
                                      + " does not match the checkpoint's vocab of "
                                      + std::to_string(model.getVocabSize()));
         }
-        gradhip::check_tokenizer_matches(model, *tokenizer, o.checkpoint);
-        const std::vector<int> prompt = tokenizer->encode(o.prompt);
+        gradhip::check_tokenizer_matches(model, *tokenizer, checkpoint);
+        const std::vector<int> prompt = tokenizer->encode(text);
         if (prompt.empty()) throw Usage("the prompt is empty");
 
         gradhip::TextGen generator(model, tokenizer.get());
         if (o.seed) generator.set_seed(*o.seed);
 
         std::cout << "\n--- Greedy Decoding ---\n" << std::endl;
-        std::cout << "Prompt: \"" << o.prompt << "\"" << std::endl;
+        std::cout << "Prompt: \"" << text << "\"" << std::endl;
         std::cout << generator.generate_greedy(prompt, o.max_tokens, o.repetition_penalty) << std::endl;
         if (o.greedy) return 0;
 
         std::cout << "\n--- Sampling (" << describe(o) << ") ---\n" << std::endl;
-        std::cout << "Prompt: \"" << o.prompt << "\"" << std::endl;
+        std::cout << "Prompt: \"" << text << "\"" << std::endl;
         std::cout << generator.generate_sample(prompt, o.temperature, o.max_tokens, o.repetition_penalty, o.top_k,
                                                o.top_p)
                   << std::endl;

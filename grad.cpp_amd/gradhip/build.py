@@ -35,7 +35,8 @@ def build(verbose: bool = True) -> str:
     subprocess.check_call(cmd)
     # the command-line caller: plain C++ over the header-only adapter
     os.makedirs(BIN_DIR, exist_ok=True)
-    for src, exe in (("generate.cpp", CLI), ("bench.cpp", os.path.join(BIN_DIR, "gradhip-bench"))):
+    for src, exe in (("generate.cpp", CLI), ("chat.cpp", os.path.join(BIN_DIR, "gradhip-chat")),
+                     ("bench.cpp", os.path.join(BIN_DIR, "gradhip-bench"))):
         cmd = ["g++", "-std=c++20", "-O2", "-Wall", "-Wextra", "-I", INCLUDE, os.path.join(PKG, "cli", src),
                "-o", exe, "-L", LIB_DIR, "-lgradhip", "-Wl,-rpath,$ORIGIN/../lib"]
         if verbose:

@@ -99,3 +99,30 @@ def test_bench_writes_the_reference_schema(tmp_path):
     assert len(rates) == 3 and all(r > 0 for r in rates)
     assert abs(j["median_generation_tokens_per_second"] - sorted(rates)[1]) < 1e-3
     assert subprocess.run([exe, "--trials", "0"], capture_output=True).returncode == 2
+
+
+def test_chat_streams_each_line(setup):
+    """gradhip-chat: `grad chat`'s loop (src/cli/chat.cpp:49-68): every line is encoded with a
+    trailing newline, echoed, and continued token by token from an empty context."""
+    d, tok, cfg, om = setup
+    exe = os.path.join(ROOT, "grad.cpp_amd", "bin", "gradhip-chat")
+    assert os.path.exists(exe), "gradhip-chat is not built; run __graft_entry__.build()"
+    lines = ["the little cat", "Once upon a time"]
+    out = subprocess.run([exe, str(d / "m.bin"), str(d / "t.tok"), "--max-tokens", "10", "--temperature", "0.9",
+                          "--top-k", "8", "--repetition-penalty", "1.15", "--seed", "5"],
+                         input=("\n".join(lines) + "\nexit\nnever read\n").encode(), capture_output=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    want = (b"\ngradhip Chat\n\n\nThis is a base language model: it continues text in the style of its training "
+            b"corpus.\nEmpty line or 'exit' quits.\n\n")
+    for line in lines:
+        ids = tok.encode((line + "\n").encode())
+        ref = O.generate_sample(om, ids, synth.uniforms(10, 5), 0.9, 10, 1.15, 8, 1.0)
+        want += b"> " + line.encode() + tok.decode(ref[len(ids):]) + b"\n\n"
+    want += b"> "
+    assert out.stdout == want
+    # --greedy is top-k 1: the arg-max stream without a draw mattering
+    out = subprocess.run([exe, str(d / "m.bin"), str(d / "t.tok"), "--max-tokens", "6", "--greedy",
+                          "--repetition-penalty", "1.0"], input=b"the cat\n\n", capture_output=True, timeout=120)
+    ids = tok.encode(b"the cat\n")
+    greedy = O.generate_greedy(om, ids, 6, 1.0)
+    assert out.returncode == 0 and b"> the cat" + tok.decode(greedy[len(ids):]) + b"\n\n> " in out.stdout
