@@ -36,7 +36,8 @@ def build(verbose: bool = True) -> str:
     # the command-line caller: plain C++ over the header-only adapter
     os.makedirs(BIN_DIR, exist_ok=True)
     for src, exe in (("generate.cpp", CLI), ("chat.cpp", os.path.join(BIN_DIR, "gradhip-chat")),
-                     ("bench.cpp", os.path.join(BIN_DIR, "gradhip-bench"))):
+                     ("bench.cpp", os.path.join(BIN_DIR, "gradhip-bench")),
+                     ("eval.cpp", os.path.join(BIN_DIR, "gradhip-eval"))):
         cmd = ["g++", "-std=c++20", "-O2", "-Wall", "-Wextra", "-I", INCLUDE, os.path.join(PKG, "cli", src),
                "-o", exe, "-L", LIB_DIR, "-lgradhip", "-Wl,-rpath,$ORIGIN/../lib"]
         if verbose:

@@ -126,3 +126,46 @@ def test_chat_streams_each_line(setup):
     ids = tok.encode(b"the cat\n")
     greedy = O.generate_greedy(om, ids, 6, 1.0)
     assert out.returncode == 0 and b"> the cat" + tok.decode(greedy[len(ids):]) + b"\n\n> " in out.stdout
+
+
+def test_eval_scores_a_token_file(setup, tmp_path):
+    """gradhip-eval: windows of a TOK1 file (src/data/token_file.cpp:149-176) in batches of eight,
+    loss as training::mean_loss forms it (src/training/trainer.cpp:319-340)."""
+    import re
+    import struct
+
+    import numpy as np
+    d, tok, cfg, om = setup
+    exe = os.path.join(ROOT, "grad.cpp_amd", "bin", "gradhip-eval")
+    assert os.path.exists(exe), "gradhip-eval is not built; run __graft_entry__.build()"
+    seq = 12
+    tokens = synth.uniform_tokens(11 * seq + 5, cfg.vocab, 71)   # 11 windows: one full batch and one of three
+    path = tmp_path / "val.bin"
+    path.write_bytes(b"TOK1" + struct.pack("<IQ", cfg.vocab, len(tokens)) + tokens.astype("<u2").tobytes())
+    out = subprocess.run([exe, str(d / "m.bin"), str(path), "--seq", str(seq)], capture_output=True, text=True,
+                         timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    m = re.search(r"^val\s+loss ([0-9.]+)  perplexity ([0-9.]+)  \((\d+) tokens, \d+s\)$", out.stdout, re.M)
+    assert m, out.stdout
+    windows = (len(tokens) - seq - 1) // seq + 1
+    assert windows == 11 and int(m.group(3)) == windows * seq
+    per_window = [O.score(om, tokens[w * seq:w * seq + seq], tokens[w * seq + 1:w * seq + seq + 1]).mean()
+                  for w in range(windows)]
+    batches = [per_window[:8], per_window[8:]]
+    want = sum(np.mean(b) * len(b) for b in batches) / windows
+    assert abs(float(m.group(1)) - want) <= 1e-3 and abs(float(m.group(2)) - np.exp(want)) <= 2e-3 * np.exp(want)
+    # --batches 1: the first batch only
+    out = subprocess.run([exe, str(d / "m.bin"), str(path), "--seq", str(seq), "--batches", "1"],
+                         capture_output=True, text=True, timeout=120)
+    m = re.search(r"loss ([0-9.]+)  perplexity [0-9.]+  \((\d+) tokens", out.stdout)
+    assert out.returncode == 0 and int(m.group(2)) == 8 * seq and abs(float(m.group(1)) - np.mean(batches[0])) <= 1e-3
+    # errors: a context longer than the model's, a file that is not a token file, the wrong vocabulary
+    out = subprocess.run([exe, str(d / "m.bin"), str(path), "--seq", "65"], capture_output=True, text=True)
+    assert out.returncode == 1 and "seq length exceeds the model's context (64)" in out.stderr
+    out = subprocess.run([exe, str(d / "m.bin"), str(d / "t.tok"), "--seq", str(seq)], capture_output=True, text=True)
+    assert out.returncode == 1 and "Not a token file (bad magic)" in out.stderr
+    other = tmp_path / "other.bin"
+    other.write_bytes(b"TOK1" + struct.pack("<IQ", cfg.vocab + 1, len(tokens)) + tokens.astype("<u2").tobytes())
+    out = subprocess.run([exe, str(d / "m.bin"), str(other), "--seq", str(seq)], capture_output=True, text=True)
+    assert out.returncode == 1 and "token files and checkpoint disagree on vocab size" in out.stderr
+    assert subprocess.run([exe, str(d / "m.bin")], capture_output=True).returncode == 2
