@@ -1329,18 +1329,19 @@ const char* gh_last_error(void) { return g_last_error.c_str(); }
 
 // ---- tokenizer (host only)
 
+// Exactly one of the two is set.
 struct gh_tokenizer {
-    gh::ByteBpe bpe;
+    std::optional<gh::ByteBpe> v2;
+    std::optional<gh::BpeV1> v1;
 };
 
 gh_status gh_tokenizer_load(const char* path, gh_tokenizer** out) {
     return guard([&] {
         if (!path || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         *out = nullptr;
-        if (!is_gtok_file(path))
-            throw ApiError{GH_ERR_RUNTIME, std::string("Tokenizer file ") + path
-                                               + ": a v1 tokenizer cache; only GTOK v2 files are supported"};
-        *out = new gh_tokenizer{ByteBpe::load(path)};
+        // anything that does not start with "GTOK" is taken for a v1 cache (tokenizer.cpp:107-117)
+        if (is_gtok_file(path)) *out = new gh_tokenizer{ByteBpe::load(path), std::nullopt};
+        else *out = new gh_tokenizer{std::nullopt, BpeV1::load(path)};
     });
 }
 
@@ -1357,14 +1358,15 @@ gh_status gh_tokenizer_from_merges(const int32_t* merges, int32_t n_merges, cons
         std::vector<std::string> sp;
         for (int32_t i = 0; i < n_specials; i++)
             sp.emplace_back(specials[i], static_cast<size_t>(std::max(special_lens[i], 0)));
-        *out = new gh_tokenizer{ByteBpe(std::move(m), std::move(sp))};
+        *out = new gh_tokenizer{ByteBpe(std::move(m), std::move(sp)), std::nullopt};
     });
 }
 
 gh_status gh_tokenizer_save(const gh_tokenizer* t, const char* path) {
     return guard([&] {
         if (!t || !path) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
-        t->bpe.save(path);
+        if (t->v2) t->v2->save(path);
+        else t->v1->save(path);
     });
 }
 
@@ -1373,19 +1375,30 @@ void gh_tokenizer_free(gh_tokenizer* t) { delete t; }
 gh_status gh_tokenizer_get_info(const gh_tokenizer* t, gh_tokenizer_info* out) {
     return guard([&] {
         if (!t || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
-        out->kind = ByteBpe::kKind;
-        out->vocab_size = t->bpe.vocab_size();
-        out->eos_id = t->bpe.special_id("<|endoftext|>");
-        out->n_merges = static_cast<int32_t>(t->bpe.merges().size());
-        out->n_specials = static_cast<int32_t>(t->bpe.specials().size());
-        out->fingerprint = t->bpe.fingerprint();
+        if (t->v2) {
+            out->kind = ByteBpe::kKind;
+            out->vocab_size = t->v2->vocab_size();
+            out->eos_id = t->v2->special_id("<|endoftext|>");  // byte_bpe.h:78
+            out->n_merges = static_cast<int32_t>(t->v2->merges().size());
+            out->n_specials = static_cast<int32_t>(t->v2->specials().size());
+            out->fingerprint = t->v2->fingerprint();
+        } else {
+            out->kind = BpeV1::kKind;
+            out->vocab_size = t->v1->vocab_size();
+            out->eos_id = t->v1->special_id("<eos>");  // tokenizer.cpp:95-97
+            out->n_merges = static_cast<int32_t>(t->v1->merge_count());
+            out->n_specials = 0;
+            for (const char* sp : {"<pad>", "<eos>", "<unk>"}) out->n_specials += t->v1->special_id(sp) >= 0;
+            out->fingerprint = t->v1->fingerprint();
+        }
     });
 }
 
 gh_status gh_tokenizer_special_id(const gh_tokenizer* t, const char* token, size_t len, int32_t* id) {
     return guard([&] {
         if (!t || !id || (len > 0 && !token)) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
-        *id = t->bpe.special_id(std::string_view(token, len));
+        const std::string_view tv(token, len);
+        *id = t->v2 ? t->v2->special_id(tv) : t->v1->special_id(tv);
     });
 }
 
@@ -1394,7 +1407,8 @@ gh_status gh_tokenizer_encode(const gh_tokenizer* t, const char* text, size_t le
     return guard([&] {
         if (!t || !n || (len > 0 && !text) || (cap > 0 && !ids))
             throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
-        const std::vector<int> got = t->bpe.encode(std::string_view(text, len), with_specials != 0);
+        const std::string_view tv(text, len);
+        const std::vector<int> got = t->v2 ? t->v2->encode(tv, with_specials != 0) : t->v1->encode(tv);
         *n = got.size();
         std::copy_n(got.begin(), std::min(cap, got.size()), ids);
     });
@@ -1405,7 +1419,7 @@ gh_status gh_tokenizer_decode(const gh_tokenizer* t, const int32_t* ids, size_t 
     return guard([&] {
         if (!t || !len || (n > 0 && !ids) || (cap > 0 && !out))
             throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
-        const std::string got = t->bpe.decode(ids, n);
+        const std::string got = t->v2 ? t->v2->decode(ids, n) : t->v1->decode(ids, n);
         *len = got.size();
         std::copy_n(got.begin(), std::min(cap, got.size()), out);
     });

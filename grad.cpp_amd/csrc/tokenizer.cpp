@@ -487,6 +487,219 @@ ByteBpe ByteBpe::load(const std::string& path) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// BpeV1
+
+namespace {
+
+constexpr std::uint64_t kMaxCacheEntries = 1u << 24;  // bpe_tokenizer.cpp:343
+constexpr std::uint64_t kMaxTokenBytes = 1u << 16;    // bpe_tokenizer.cpp:344
+
+std::string pair_string(const std::string& left, const std::string& right) {
+    std::string key;
+    key.reserve(left.size() + right.size() + 1);
+    key += left;
+    key += '\0';
+    key += right;
+    return key;
+}
+
+// Cache fields are the writer's host types: 64-bit size_t, 32-bit int, little endian.
+std::uint64_t cache_u64(std::istream& in, const std::string& path, const char* what) {
+    unsigned char b[8];
+    in.read(reinterpret_cast<char*>(b), 8);
+    if (!in) throw std::runtime_error("Tokenizer cache truncated reading " + std::string(what) + ": " + path);
+    std::uint64_t v = 0;
+    for (int i = 7; i >= 0; i--) v = (v << 8) | b[i];
+    return v;
+}
+
+std::string cache_token(std::istream& in, const std::string& path) {
+    const std::uint64_t len = cache_u64(in, path, "token length");
+    if (len > kMaxTokenBytes)
+        throw std::runtime_error("Tokenizer cache has an implausible token length (" + std::to_string(len)
+                                 + " bytes): " + path);
+    std::string token(len, '\0');
+    in.read(token.data(), static_cast<std::streamsize>(len));
+    if (!in) throw std::runtime_error("Tokenizer cache truncated reading a token: " + path);
+    return token;
+}
+
+bool c_space(char c) { return c == ' ' || (c >= '\t' && c <= '\r'); }  // what `stream >> word` skips
+
+}  // namespace
+
+BpeV1::BpeV1(std::vector<std::pair<std::string, int>> vocab, std::vector<Merge> merges)
+    : merges_(std::move(merges)) {
+    for (auto& [token, id] : vocab) {
+        id_to_token_[id] = token;
+        vocab_[std::move(token)] = id;
+    }
+    for (std::size_t r = 0; r < merges_.size(); r++)
+        ranks_[pair_string(merges_[r].first, merges_[r].second)].push_back(static_cast<int>(r));
+
+    // v1_fingerprint (tokenizer.cpp:39-60): the id-ordered token table, then the merges
+    std::vector<std::pair<int, const std::string*>> by_id;
+    by_id.reserve(id_to_token_.size());
+    for (const auto& [id, token] : id_to_token_) by_id.emplace_back(id, &token);
+    std::sort(by_id.begin(), by_id.end(), [](const auto& a, const auto& b) { return a.first < b.first; });
+    Fnv1a64 h;
+    h.str("grad.tokenizer.bpe_v1");
+    h.u32(static_cast<std::uint32_t>(by_id.size()));
+    for (const auto& [id, token] : by_id) {
+        h.u32(static_cast<std::uint32_t>(id));
+        h.str(*token);
+    }
+    h.u32(static_cast<std::uint32_t>(merges_.size()));
+    for (const Merge& m : merges_) {
+        h.str(m.first);
+        h.str(m.second);
+    }
+    fingerprint_ = h.value();
+}
+
+BpeV1 BpeV1::load(const std::string& path) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) throw std::runtime_error("Failed to open file for loading: " + path);
+    const std::uint64_t n_vocab = cache_u64(f, path, "vocab size");
+    if (n_vocab > kMaxCacheEntries)
+        throw std::runtime_error("Tokenizer cache has an implausible vocab size (" + std::to_string(n_vocab)
+                                 + "): " + path);
+    std::vector<std::pair<std::string, int>> vocab;
+    vocab.reserve(n_vocab);
+    for (std::uint64_t i = 0; i < n_vocab; i++) {
+        std::string token = cache_token(f, path);
+        unsigned char b[4];
+        f.read(reinterpret_cast<char*>(b), 4);
+        if (!f) throw std::runtime_error("Tokenizer cache truncated reading token id: " + path);
+        const auto id = static_cast<std::int32_t>(b[0] | (std::uint32_t{b[1]} << 8) | (std::uint32_t{b[2]} << 16)
+                                                  | (std::uint32_t{b[3]} << 24));
+        if (id < 0) throw std::runtime_error("Tokenizer cache has a negative token id: " + path);
+        vocab.emplace_back(std::move(token), id);
+    }
+    const std::uint64_t n_merges = cache_u64(f, path, "merge count");
+    if (n_merges > kMaxCacheEntries)
+        throw std::runtime_error("Tokenizer cache has an implausible merge count (" + std::to_string(n_merges)
+                                 + "): " + path);
+    std::vector<Merge> merges;
+    merges.reserve(n_merges);
+    for (std::uint64_t i = 0; i < n_merges; i++) {
+        std::string left = cache_token(f, path);
+        std::string right = cache_token(f, path);
+        merges.emplace_back(std::move(left), std::move(right));
+    }
+    return BpeV1(std::move(vocab), std::move(merges));
+}
+
+void BpeV1::save(const std::string& path) const {
+    std::string buf;
+    const auto token = [&](const std::string& t) {
+        put_u64(buf, t.size());
+        buf += t;
+    };
+    std::vector<std::pair<int, const std::string*>> by_id;
+    for (const auto& [t, id] : vocab_) by_id.emplace_back(id, &t);
+    std::sort(by_id.begin(), by_id.end(), [](const auto& a, const auto& b) { return a.first < b.first; });
+    put_u64(buf, by_id.size());
+    for (const auto& [id, t] : by_id) {
+        token(*t);
+        put_u32(buf, static_cast<std::uint32_t>(id));
+    }
+    put_u64(buf, merges_.size());
+    for (const Merge& m : merges_) {
+        token(m.first);
+        token(m.second);
+    }
+    std::ofstream f(path, std::ios::binary);
+    if (!f) throw std::runtime_error("Failed to open file for saving: " + path);
+    f.write(buf.data(), static_cast<std::streamsize>(buf.size()));
+    f.close();
+    if (!f) throw std::runtime_error("Failed while writing tokenizer cache: " + path);
+}
+
+int BpeV1::special_id(std::string_view token) const {
+    if (token != "<pad>" && token != "<eos>" && token != "<unk>") return -1;
+    const auto it = vocab_.find(std::string(token));
+    return it == vocab_.end() ? -1 : it->second;
+}
+
+// The merge list is walked once, in order, and a merge joins every occurrence of
+// its pair from left to right (bpe_tokenizer.cpp:222-247).  Instead of testing
+// all merges against the word, the next merge to act is the lowest rank, at or
+// after the last one applied, among the pairs the word holds now.
+void BpeV1::encode_word(const std::string& word, std::vector<int>& out) const {
+    std::vector<std::string> parts;
+    parts.reserve(word.size());
+    for (const char c : word) parts.emplace_back(1, c);
+    int from = 0;
+    while (parts.size() > 1) {
+        int best = INT_MAX;
+        for (std::size_t i = 0; i + 1 < parts.size(); i++) {
+            const auto it = ranks_.find(pair_string(parts[i], parts[i + 1]));
+            if (it == ranks_.end()) continue;
+            const auto r = std::lower_bound(it->second.begin(), it->second.end(), from);
+            if (r != it->second.end()) best = std::min(best, *r);
+        }
+        if (best == INT_MAX) break;
+        const Merge& m = merges_[static_cast<std::size_t>(best)];
+        std::vector<std::string> next;
+        next.reserve(parts.size());
+        for (std::size_t i = 0; i < parts.size(); i++) {
+            if (i + 1 < parts.size() && parts[i] == m.first && parts[i + 1] == m.second) {
+                next.push_back(m.first + m.second);
+                i++;
+            } else {
+                next.push_back(std::move(parts[i]));
+            }
+        }
+        parts = std::move(next);
+        from = best + 1;
+    }
+    for (const std::string& p : parts) {
+        const auto it = vocab_.find(p);
+        out.push_back(it == vocab_.end() ? 2 : it->second);  // unk_token_id, bpe_tokenizer.h:30
+    }
+}
+
+std::vector<int> BpeV1::encode(std::string_view text) const {
+    std::vector<int> out;
+    std::unordered_map<std::string, std::pair<std::size_t, std::size_t>> seen;
+    bool first = true;
+    for (std::size_t pos = 0; pos < text.size();) {
+        while (pos < text.size() && c_space(text[pos])) pos++;
+        std::size_t end = pos;
+        while (end < text.size() && !c_space(text[end])) end++;
+        if (end == pos) break;
+        std::string word = first ? std::string() : std::string("_");
+        word.append(text.substr(pos, end - pos));
+        first = false;
+        pos = end;
+        if (const auto hit = seen.find(word); hit != seen.end()) {
+            // out may reallocate while it grows: copy through indices
+            for (std::size_t i = 0; i < hit->second.second; i++) {
+                const int id = out[hit->second.first + i];
+                out.push_back(id);
+            }
+            continue;
+        }
+        const std::size_t before = out.size();
+        encode_word(word, out);
+        seen.emplace(std::move(word), std::make_pair(before, out.size() - before));
+    }
+    return out;
+}
+
+std::string BpeV1::decode(const int* ids, std::size_t n) const {
+    std::string out;
+    for (std::size_t i = 0; i < n; i++) {
+        const auto it = id_to_token_.find(ids[i]);
+        if (it != id_to_token_.end()) out += it->second;
+    }
+    for (char& c : out)
+        if (c == '_') c = ' ';
+    return out;
+}
+
 bool is_gtok_file(const std::string& path) {
     std::ifstream f(path, std::ios::binary);
     if (!f) throw std::runtime_error("Failed to open tokenizer file: " + path);

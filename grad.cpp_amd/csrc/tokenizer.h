@@ -96,6 +96,46 @@ private:
     std::uint64_t fingerprint_ = 0;
 };
 
+// The original whitespace BPE (grad::BPETokenizer behind grad::BpeV1,
+// include/grad/tokenizer/bpe_tokenizer.h:21-55, src/tokenizer/bpe_tokenizer.cpp): text is
+// split at white space, every word but the first gets a leading '_', a word's
+// characters are joined by the merge list in order, strings missing from the
+// vocabulary become <unk>; decode turns every '_' into a space, so it is lossy.
+class BpeV1 {
+public:
+    static constexpr std::uint32_t kKind = 1;  // fingerprint.h: TokenizerKind::BpeV1
+    using Merge = std::pair<std::string, std::string>;
+
+    // vocab: (token string, id) in any order, as the cache stores them.
+    BpeV1(std::vector<std::pair<std::string, int>> vocab, std::vector<Merge> merges);
+    // Reads a tokenizer cache (bpe_tokenizer.cpp:373-417): host size_t and int
+    // fields as an x86-64 / AArch64 Linux build writes them (8 and 4 bytes, little
+    // endian).  Throws std::runtime_error with BPETokenizer::load's messages.
+    static BpeV1 load(const std::string& path);
+    // Entries in id order (grad.cpp writes its hash map's order; it reads any order).
+    void save(const std::string& path) const;
+
+    std::vector<int> encode(std::string_view text) const;
+    std::string decode(const int* ids, std::size_t n) const;  // unknown ids are skipped
+
+    int vocab_size() const { return static_cast<int>(vocab_.size()); }  // getCurrentVocabSize
+    // "<pad>", "<eos>" and "<unk>" when the vocabulary has them (tokenizer.cpp:99-104); else -1.
+    int special_id(std::string_view token) const;
+    std::uint64_t fingerprint() const { return fingerprint_; }  // tokenizer.cpp:39-60
+    std::size_t merge_count() const { return merges_.size(); }
+
+private:
+    void encode_word(const std::string& word, std::vector<int>& out) const;
+
+    std::unordered_map<std::string, int> vocab_;
+    std::unordered_map<int, std::string> id_to_token_;
+    std::vector<Merge> merges_;
+    // (left, right) -> ranks in the merge list, ascending; '\0' cannot occur in a
+    // word, so it separates the two strings of a key
+    std::unordered_map<std::string, std::vector<int>> ranks_;
+    std::uint64_t fingerprint_ = 0;
+};
+
 // True when the file starts with "GTOK" (tokenizer.cpp: detect_tokenizer_file);
 // throws std::runtime_error("Failed to open tokenizer file: <path>").
 bool is_gtok_file(const std::string& path);

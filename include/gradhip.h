@@ -204,18 +204,18 @@ gh_status gh_session_generate(gh_session* s, const int32_t* prompts, int32_t pro
 typedef struct gh_tokenizer gh_tokenizer;
 
 typedef struct gh_tokenizer_info {
-    uint32_t kind;        /* TokenizerKind, fingerprint.h:15-18: 2 = byte-level BPE */
+    uint32_t kind;        /* TokenizerKind, fingerprint.h:15-18: 1 = v1 whitespace BPE, 2 = byte-level BPE */
     int32_t vocab_size;   /* Tokenizer::vocab_size */
-    int32_t eos_id;       /* Tokenizer::eos_id ("<|endoftext|>"), -1 when absent */
+    int32_t eos_id;       /* Tokenizer::eos_id ("<|endoftext|>"; "<eos>" for v1), -1 when absent */
     int32_t n_merges;
     int32_t n_specials;
     uint64_t fingerprint; /* Tokenizer::fingerprint; what a checkpoint's TKFP trailer records */
 } gh_tokenizer_info;
 
-/* load_tokenizer (tokenizer.h:52, tokenizer.cpp:119-124): opens a "GTOK" v2 file
- * (ByteBpe::load, byte_bpe.cpp:676-744) with the same validation and messages.
- * A file that does not start with "GTOK" is a v1 cache in grad.cpp; those are
- * refused here with GH_ERR_RUNTIME. */
+/* load_tokenizer (tokenizer.h:52, tokenizer.cpp:119-124): a file that starts
+ * with "GTOK" is a v2 file (ByteBpe::load, byte_bpe.cpp:676-744), anything else
+ * is taken for a v1 cache (BPETokenizer::load, bpe_tokenizer.cpp:373-417, with
+ * 64-bit size_t and 32-bit int fields); same validation and messages. */
 gh_status gh_tokenizer_load(const char* path, gh_tokenizer** out);
 /* ByteBpe(merges, specials) (byte_bpe.h:50-53): merges is n_merges x 2 ids;
  * specials[i] has special_lens[i] bytes.  GH_ERR_INVALID_ARGUMENT with the
@@ -229,7 +229,7 @@ gh_status gh_tokenizer_get_info(const gh_tokenizer* t, gh_tokenizer_info* out);
 /* Tokenizer::special_id (tokenizer.h:33): *id = -1 when token is not special. */
 gh_status gh_tokenizer_special_id(const gh_tokenizer* t, const char* token, size_t len, int32_t* id);
 /* Tokenizer::encode (with_specials != 0) / ByteBpe::encode_ordinary (== 0),
- * byte_bpe.cpp:555-591.  *n receives the number of ids of the whole text; at
+ * byte_bpe.cpp:555-591; a v1 tokenizer has one encoding (bpe_tokenizer.cpp:175-270).  *n receives the number of ids of the whole text; at
  * most cap of them are written to ids (call with cap = 0 to size a buffer). */
 gh_status gh_tokenizer_encode(const gh_tokenizer* t, const char* text, size_t len, int32_t with_specials,
                               int32_t* ids, size_t cap, size_t* n);

@@ -9,8 +9,8 @@
 //     grad::InferenceSession          -> gradhip::InferenceSession    (inference.h:16-29)
 //     grad::TextGen                   -> gradhip::TextGen             (text_gen.h:12-38)
 //     grad::Tokenizer                 -> gradhip::Tokenizer           (tokenizer.h:20-43)
-//     grad::ByteBpe, load_tokenizer   -> gradhip::ByteBpe, gradhip::load_tokenizer
-//                                                                      (byte_bpe.h:37-113, tokenizer.h:52)
+//     grad::ByteBpe, grad::BpeV1,     -> gradhip::ByteBpe, gradhip::BpeV1, gradhip::load_tokenizer
+//     load_tokenizer                                                   (byte_bpe.h:37-113, bpe_v1.h, tokenizer.h:52)
 //
 // The model lives on the GPU; there is no CPU path behind these classes.
 #pragma once
@@ -113,7 +113,9 @@ public:
     [[nodiscard]] static ByteBpe load(const std::string& path) {
         gh_tokenizer* t = nullptr;
         check(gh_tokenizer_load(path.c_str(), &t));
-        return ByteBpe(t);
+        ByteBpe out(t);
+        if (out.info_.kind != 2) throw std::runtime_error("Tokenizer file " + path + ": not a GTOK tokenizer file");
+        return out;
     }
     ByteBpe(const ByteBpe&) = delete;
     ByteBpe& operator=(const ByteBpe&) = delete;
@@ -156,9 +158,67 @@ private:
     gh_tokenizer_info info_{};
 };
 
-// load_tokenizer (tokenizer.h:52).  grad.cpp also opens v1 caches here; this
-// library reads "GTOK" files only and throws std::runtime_error for anything else.
+// grad::BpeV1 (bpe_v1.h) without the trainer: the original whitespace BPE read
+// from a tokenizer cache.  decode is lossy ('_' and white-space runs read back as
+// one space); ids missing from the vocabulary are skipped.
+class BpeV1 final : public Tokenizer {
+public:
+    // Throws std::runtime_error with BPETokenizer::load's messages (bpe_tokenizer.cpp:373-417).
+    [[nodiscard]] static BpeV1 load(const std::string& path) {
+        gh_tokenizer* t = nullptr;
+        check(gh_tokenizer_load(path.c_str(), &t));
+        BpeV1 out(t);
+        if (out.info_.kind != 1) throw std::runtime_error(path + " holds a v2 tokenizer, not v1");
+        return out;
+    }
+    BpeV1(const BpeV1&) = delete;
+    BpeV1& operator=(const BpeV1&) = delete;
+    BpeV1(BpeV1&& o) noexcept : t_(std::exchange(o.t_, nullptr)), info_(o.info_) {}
+    ~BpeV1() override { gh_tokenizer_free(t_); }
+
+    [[nodiscard]] TokenizerKind kind() const override { return TokenizerKind::BpeV1; }
+    [[nodiscard]] std::vector<int> encode(std::string_view text) const override {
+        std::vector<int> ids(text.size());  // at most one id per byte
+        std::size_t n = 0;
+        check(gh_tokenizer_encode(t_, text.data(), text.size(), 1, ids.data(), ids.size(), &n));
+        ids.resize(n);
+        return ids;
+    }
+    [[nodiscard]] std::string decode(std::span<const int> ids) const override {
+        std::size_t len = 0;
+        check(gh_tokenizer_decode(t_, ids.data(), ids.size(), nullptr, 0, &len));
+        std::string out(len, '\0');
+        check(gh_tokenizer_decode(t_, ids.data(), ids.size(), out.data(), out.size(), &len));
+        return out;
+    }
+    [[nodiscard]] int vocab_size() const override { return info_.vocab_size; }
+    [[nodiscard]] std::optional<int> eos_id() const override {
+        return info_.eos_id < 0 ? std::nullopt : std::optional<int>(info_.eos_id);
+    }
+    [[nodiscard]] std::optional<int> special_id(std::string_view token) const override {
+        int32_t id = -1;
+        check(gh_tokenizer_special_id(t_, token.data(), token.size(), &id));
+        return id < 0 ? std::nullopt : std::optional<int>(id);
+    }
+    [[nodiscard]] std::uint64_t fingerprint() const override { return info_.fingerprint; }
+    void save(const std::string& path) const override { check(gh_tokenizer_save(t_, path.c_str())); }
+
+private:
+    explicit BpeV1(gh_tokenizer* t) : t_(t) { check(gh_tokenizer_get_info(t_, &info_)); }
+    gh_tokenizer* t_ = nullptr;
+    gh_tokenizer_info info_{};
+};
+
+// load_tokenizer (tokenizer.h:52, tokenizer.cpp:119-124): a "GTOK" file is the
+// byte-level BPE, anything else is taken for a v1 cache.
 [[nodiscard]] inline std::unique_ptr<Tokenizer> load_tokenizer(const std::string& path) {
+    gh_tokenizer* t = nullptr;
+    check(gh_tokenizer_load(path.c_str(), &t));
+    gh_tokenizer_info info{};
+    const gh_status st = gh_tokenizer_get_info(t, &info);
+    gh_tokenizer_free(t);
+    check(st);
+    if (info.kind == 1) return std::make_unique<BpeV1>(BpeV1::load(path));
     return std::make_unique<ByteBpe>(ByteBpe::load(path));
 }
 

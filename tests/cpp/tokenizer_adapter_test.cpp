@@ -44,6 +44,21 @@ int main(int argc, char** argv) {
         }
         const gradhip::ByteBpe tiny({{97, 98}});
         std::printf("tiny %s\n", gradhip::to_string(tiny.identity()).c_str());
+        if (argc >= 4) {  // a v1 cache through the same loader
+            const std::unique_ptr<gradhip::Tokenizer> v1 = gradhip::load_tokenizer(argv[3]);
+            std::printf("v1 %s vocab %d eos %d unk %d\n", gradhip::to_string(v1->identity()).c_str(), v1->vocab_size(),
+                        v1->eos_id().value_or(-1), v1->special_id("<unk>").value_or(-1));
+            const std::vector<int> v1_ids = v1->encode(text);
+            std::printf("v1ids");
+            for (int id : v1_ids) std::printf(" %d", id);
+            std::printf("\nv1text %s\n", v1->decode(v1_ids).c_str());
+            try {
+                (void)gradhip::ByteBpe::load(argv[3]);
+                std::printf("error none\n");
+            } catch (const std::runtime_error& e) {
+                std::printf("runtime_error %s\n", e.what());
+            }
+        }
     } catch (const std::exception& e) {
         std::printf("FATAL %s\n", e.what());
         return 1;

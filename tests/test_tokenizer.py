@@ -267,8 +267,10 @@ def test_corrupt_files(tmp_path):
     assert changed in ("fingerprint does not match the contents (corrupt file)",) or "repeats an earlier merge" in changed
     flipped = good[:-1] + bytes([good[-1] ^ 1])
     assert why(flipped) == "fingerprint does not match the contents (corrupt file)"
-    # a file that does not start with the magic is a v1 cache in grad.cpp: refused here
-    assert "v1 tokenizer cache" in why(b"GTOX" + good[4:])
+    # a file that does not start with the magic is taken for a v1 cache (tokenizer.cpp:107-124)
+    bad.write_bytes(b"GTOX" + good[4:])
+    with pytest.raises(RuntimeError, match="Tokenizer cache has an implausible vocab size"):
+        G.Tokenizer.load(bad)
     with pytest.raises(RuntimeError, match="Failed to open tokenizer file: "):
         G.Tokenizer.load(tmp_path / "missing.tok")
 

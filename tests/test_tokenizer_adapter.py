@@ -21,6 +21,17 @@ def test_cpp_tokenizer_caller_matches_the_oracle(tmp_path):
     ref = R.train((text * 3 + "the cat sat on the mat and the cat ran to the hat\n" * 5).encode(), 330)
     path = tmp_path / "t.tok"
     path.write_bytes(ref.file_image())
+    v1 = R.train_v1(text.replace("\n", " ").encode() * 3, 120)
+    v1_path = tmp_path / "v1.cache"
+    v1_path.write_bytes(v1.cache_image())
+    one_line = "Once upon a time,   the little_cat said"
+    out = subprocess.run([exe, str(path), one_line, str(v1_path)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stdout + out.stderr
+    lines = out.stdout.strip().split("\n")
+    assert lines[9] == f"v1 v1:{v1.fingerprint():016x} vocab {v1.vocab_size} eos 1 unk 2"
+    assert [int(x) for x in lines[10].split()[1:]] == v1.encode(one_line.encode())
+    assert lines[11] == "v1text Once upon a time, the little cat said"
+    assert lines[12] == f"runtime_error Tokenizer file {v1_path}: not a GTOK tokenizer file"
     out = subprocess.run([exe, str(path), text], capture_output=True, text=True, timeout=60)
     assert out.returncode == 0, out.stdout + out.stderr
     lines = out.stdout.strip().split("\n")
