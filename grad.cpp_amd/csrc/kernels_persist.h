@@ -543,29 +543,38 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                         m = mn;
                     }
                 }
-                // every lane group (16 lanes = one position slot) leaves its share; the
-                // groups of a wavefront share its running maximum
-                float* mine = part + (wave * 4 + sub) * 68;
-                reinterpret_cast<float4*>(mine + 4)[dl] = acc;
-                if (dl == 0) {
-                    mine[0] = m;
-                    mine[1] = lsum;
+                // The four lane groups of a wavefront (16 lanes = one position slot each)
+                // share its running maximum: their sums are added across the groups, and
+                // the wavefront leaves one share.
+                lsum += __shfl_xor(lsum, 16, kWave);
+                acc.x += __shfl_xor(acc.x, 16, kWave);
+                acc.y += __shfl_xor(acc.y, 16, kWave);
+                acc.z += __shfl_xor(acc.z, 16, kWave);
+                acc.w += __shfl_xor(acc.w, 16, kWave);
+                lsum += __shfl_xor(lsum, 32, kWave);
+                acc.x += __shfl_xor(acc.x, 32, kWave);
+                acc.y += __shfl_xor(acc.y, 32, kWave);
+                acc.z += __shfl_xor(acc.z, 32, kWave);
+                acc.w += __shfl_xor(acc.w, 32, kWave);
+                float* mine = part + wave * 68;  // m, l, pad, pad, acc[64]
+                if (sub == 0) {
+                    reinterpret_cast<float4*>(mine + 4)[dl] = acc;
+                    if (dl == 0) {
+                        mine[0] = m;
+                        mine[1] = lsum;
+                    }
                 }
                 __syncthreads();
                 if (tid < HS) {
                     float M = -INFINITY;
-                    for (int w8 = 0; w8 < kPersistWaves; w8++) M = fmaxf(M, part[w8 * 4 * 68]);
-                    float Lsum = 0.0f, o = 0.0f;
-                    for (int w8 = 0; w8 < kPersistWaves; w8++) {
-                        const float f = expf(part[w8 * 4 * 68] - M);  // 0 for wavefronts without positions
-                        float ls = 0.0f, os = 0.0f;
 #pragma unroll
-                        for (int g4 = 0; g4 < 4; g4++) {
-                            ls += part[(w8 * 4 + g4) * 68 + 1];
-                            os += part[(w8 * 4 + g4) * 68 + 4 + tid];
-                        }
-                        Lsum += ls * f;
-                        o += os * f;
+                    for (int w8 = 0; w8 < kPersistWaves; w8++) M = fmaxf(M, part[w8 * 68]);
+                    float Lsum = 0.0f, o = 0.0f;
+#pragma unroll
+                    for (int w8 = 0; w8 < kPersistWaves; w8++) {
+                        const float f = expf(part[w8 * 68] - M);  // 0 for wavefronts without positions
+                        Lsum += part[w8 * 68 + 1] * f;
+                        o += part[w8 * 68 + 4 + tid] * f;
                     }
                     cell_put(p.at + hd * HS + tid, o * (1.0f / Lsum), tag_of(l, 1));
                 }
