@@ -134,6 +134,11 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
     if (blockIdx.x != 0) return true;
     const int tid = threadIdx.x;
     if (p.prof && i_pick < 1024 && tid == 0) p.prof[p.prof_cap / 2 + 4 * i_pick + 2] = __builtin_amdgcn_s_memrealtime();
+    PickParams pk = p.pick;
+    pk.n_hist = p.pick.n_hist + i_pick;
+    pk.pick_idx = p.pick.pick_idx + i_pick;
+    // the draw needs no logits: form it while they arrive
+    const float u = pk.greedy ? 0.0f : pick_draw(pk, 0);
     if (wait_logits) {
         // one wavefront watches the 16 arrival counters; the workgroup meets once
         bool failed = false;
@@ -166,11 +171,8 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
     }
     unsigned long long* pp = (p.prof && i_pick < 1024) ? p.prof + p.prof_cap / 2 + 4 * i_pick : nullptr;
     if (pp && tid == 0) pp[0] = __builtin_amdgcn_s_memrealtime();
-    PickParams pk = p.pick;
-    pk.n_hist = p.pick.n_hist + i_pick;
-    pk.pick_idx = p.pick.pick_idx + i_pick;
-    const int chosen = ROW_LDS ? pick_body<true, kPersistThreads>(pk, 0, lds, lds + pk.V)
-                               : pick_body<true, kPersistThreads>(pk, 0, pk.work, lds);
+    const int chosen = ROW_LDS ? pick_body<true, kPersistThreads>(pk, 0, lds, lds + pk.V, u)
+                               : pick_body<true, kPersistThreads>(pk, 0, pk.work, lds, u);
     if (tid == 0) {
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         cell_put(p.tokc, __int_as_float(chosen), tok_tag);

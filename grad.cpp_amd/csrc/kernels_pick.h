@@ -666,8 +666,20 @@ __device__ inline float top_p_cutoff(const float* val, int V, float top_p, float
 // NT: threads of the workgroup.
 // Always inlined: each call site knows whether val is LDS or global memory, and
 // the row's loads and stores are compiled for that address space.
+// The uniform draw of pick p.pick_idx of sequence b: the caller's, or word
+// pick_idx of the Philox stream keyed by (seed, sequence), as a 24-bit fraction.
+__device__ __forceinline__ float pick_draw(const PickParams& p, int b) {
+    if (p.uniforms) return p.uniforms[static_cast<size_t>(b) * p.u_stride + p.pick_idx];
+    const unsigned w = philox4x32_10(static_cast<unsigned>(p.pick_idx) >> 2, static_cast<unsigned>(p.pick_idx) & 3u,
+                                     p.seed_lo, p.seed_hi ^ static_cast<unsigned>(b));
+    return static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
+}
+
+// u_ready: the draw when the caller has already formed it (it does not depend on
+// the logits, so it can be had while they are still on their way); negative: form it here.
 template <bool coherent, int NT>
-__device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val, float* srt) {
+__device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val, float* srt,
+                                         float u_ready = -1.0f) {
     __shared__ float red[kPickThreads / 64];
     __shared__ int redi[kPickThreads / 64];
     __shared__ unsigned hist256[256];
@@ -786,15 +798,7 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
     } else {
         // ---- sample_from_logits (text_gen.cpp:135-209)
         const float inv_t = 1.0f / p.temperature;
-        float u;
-        if (p.uniforms) {
-            u = p.uniforms[static_cast<size_t>(b) * p.u_stride + p.pick_idx];
-        } else {
-            const unsigned w = philox4x32_10(static_cast<unsigned>(p.pick_idx) >> 2,
-                                             static_cast<unsigned>(p.pick_idx) & 3u, p.seed_lo,
-                                             p.seed_hi ^ static_cast<unsigned>(b));
-            u = static_cast<float>(w >> 8) * (1.0f / 16777216.0f);
-        }
+        const float u = u_ready >= 0.0f ? u_ready : pick_draw(p, b);
         // elements per thread when a thread keeps its share of the row in registers
         const int per_thread = (V + nt - 1) / nt;
         if (p.top_k > 0 && p.top_k <= 64 && p.top_k < V && p.sort_cap >= kFastLdsFloats && per_thread <= 64) {
