@@ -33,7 +33,6 @@ struct PickParams {
     int u_stride;
     unsigned seed_lo, seed_hi;
     int sort_cap;  // floats of LDS work area next to (or instead of) the row
-    int* err;
 };
 
 // LDS work area of the pick: the small-k selection wants two floats per thread
