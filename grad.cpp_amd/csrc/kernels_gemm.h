@@ -95,6 +95,26 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
     for (int t = 0; t < MT; t++)
         ap[t] = p.in + static_cast<size_t>(min(m0 + t * 16 + fr, M - 1)) * p.in_stride + wave * kq + fc * 4;
     const float* gp = RMS ? p.gamma + wave * kq + g * 4 : nullptr;
+    // The first pair of outputs this thread will finish: what its epilogue reads
+    // (bias, residual, position, page, rotation) is requested now, not after the
+    // products, where it would be one or two more trips to memory on the tail.
+    constexpr int kEpiElems = MT * NT * 128;
+    const auto epi_at = [&](int e, int& m, int& n, int& tile_t, int& tile_u, int& at) {
+        const int tile = e >> 7, rem = e & 127;
+        tile_t = tile / NT;
+        tile_u = tile % NT;
+        const int i = rem >> 3, jp = (rem & 7) * 2;
+        m = m0 + tile_t * 16 + i;
+        n = n0 + tile_u * 16 + jp;
+        at = i * 16 + jp;
+    };
+    EpiOperands first_epi;
+    {
+        int m, n, t, u, at;
+        epi_at(static_cast<int>(threadIdx.x), m, n, t, u, at);
+        if (static_cast<int>(threadIdx.x) < kEpiElems && m < M && n < p.N)
+            first_epi = epi_fetch<EPI>(p, m, n, n + 1 < p.N);
+    }
     v4f acc[MT][NT];
     float ss[MT];
 #pragma unroll
@@ -171,13 +191,11 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
     }
     __syncthreads();
     // Column pairs (n, n+1) of one row go through the shared epilogue.
-    for (int e = threadIdx.x; e < MT * NT * 128; e += 64 * KW) {
-        const int tile = e >> 7, rem = e & 127;
-        const int t = tile / NT, u = tile % NT;
-        const int i = rem >> 3, jp = (rem & 7) * 2;
-        const int m = m0 + t * 16 + i, n = n0 + u * 16 + jp;
+    for (int e = threadIdx.x; e < kEpiElems; e += 64 * KW) {
+        int m, n, t, u, at;
+        epi_at(e, m, n, t, u, at);
         if (m >= M || n >= p.N) continue;
-        const int at = i * 16 + jp;
+        const int i = at >> 4;
         float v0 = 0.0f, v1 = 0.0f;
 #pragma unroll
         for (int w = 0; w < KW; w++) {
@@ -192,7 +210,9 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
             v0 *= r;
             v1 *= r;
         }
-        gemv_epilogue<EPI>(p, m, n, v0, v1, n + 1 < p.N);
+        const bool has1 = n + 1 < p.N;
+        if (e == static_cast<int>(threadIdx.x)) epi_apply<EPI>(p, m, n, v0, v1, has1, first_epi);
+        else gemv_epilogue<EPI>(p, m, n, v0, v1, has1);
     }
 }
 

@@ -43,9 +43,62 @@ struct GemvParams {
     int pos_base;
 };
 
+// What the epilogue of one pair of outputs (row, row + 1) of input row b needs
+// from memory besides the two products.  Fetching it is separate from applying
+// it so that a kernel can issue these loads before its main loop: they do not
+// depend on the products, and left to the end they are one or two more trips to
+// memory on the tail of every launch (position -> page table and rotation
+// tables -> store).
+struct EpiOperands {
+    float b0 = 0.0f, b1 = 0.0f;  // bias pair
+    float r0 = 0.0f, r1 = 0.0f;  // EPI_RESID: the outputs' current values
+    float cs = 1.0f, sn = 0.0f;  // EPI_QKV: rotation of the pair
+    int pos = 0, seq = 0, page = 0;  // EPI_QKV: position, sequence, physical cache page
+};
+
+template <int EPI>
+__device__ __forceinline__ EpiOperands epi_fetch(const GemvParams& p, int b, int row, bool has1) {
+    EpiOperands o;
+    if constexpr (EPI == EPI_STORE || EPI == EPI_RESID) {
+        if (p.bias) {
+            o.b0 = p.bias[row];
+            if (has1) o.b1 = p.bias[row + 1];
+        }
+    }
+    if constexpr (EPI == EPI_RESID) {
+        const float* cur = p.out + static_cast<size_t>(b) * p.out_stride;
+        o.r0 = cur[row];
+        if (has1) o.r1 = cur[row + 1];
+    }
+    if constexpr (EPI == EPI_GELU || EPI == EPI_QKV) {
+        o.b0 = p.bias[row];
+        if (has1) o.b1 = p.bias[row + 1];
+    }
+    if constexpr (EPI == EPI_QKV) {
+        // rows_per_seq == 0: one row per sequence, all at st->pos (a decode step)
+        o.seq = b;
+        if (p.rows_per_seq > 0) {
+            o.seq = b / p.rows_per_seq;
+            o.pos = p.pos_base + (b - o.seq * p.rows_per_seq);
+        } else {
+            o.pos = p.st->pos;
+        }
+        if (p.rope && row < 2 * p.d_model) {
+            // head_size is even under RoPE, so (row, row+1) is one rotation pair.
+            const int hs = p.kv.head_size;
+            const int j = ((row % p.d_model) % hs) >> 1;
+            o.cs = p.rope_cos[o.pos * (hs >> 1) + j];
+            o.sn = p.rope_sin[o.pos * (hs >> 1) + j];
+        }
+        // row + 1 may already be a key row when d_model is odd
+        if (row + 1 >= p.d_model) o.page = p.kv.page_table[o.seq * p.kv.pages_per_seq + (o.pos >> p.kv.page_shift)];
+    }
+    return o;
+}
+
 // One projected value of the fused QKV product goes to the q buffer or straight
 // into the cache row of the current position (inference.cpp:195-199).
-__device__ __forceinline__ void store_qkv(const GemvParams& p, int m, int seq, int row, float v, int pos) {
+__device__ __forceinline__ void store_qkv(const GemvParams& p, int m, int row, float v, const EpiOperands& o) {
     const int d = p.d_model;
     const int sec = row / d, c = row - sec * d;
     if (sec == 0) {
@@ -53,54 +106,51 @@ __device__ __forceinline__ void store_qkv(const GemvParams& p, int m, int seq, i
     } else {
         const int hs = p.kv.head_size;
         const int head = c / hs, j = c - head * hs;
-        p.kv.pool[kv_offset(p.kv, p.layer, seq, sec - 1, head, pos) + j] = v;
+        const int slot = o.pos & ((1 << p.kv.page_shift) - 1);
+        const size_t run =
+            (((static_cast<size_t>(p.layer) * p.kv.n_pages + o.page) * 2 + (sec - 1)) * p.kv.heads + head);
+        p.kv.pool[((run << p.kv.page_shift) + slot) * hs + j] = v;
+    }
+}
+
+template <int EPI>
+__device__ __forceinline__ void epi_apply(const GemvParams& p, int b, int row, float v0, float v1, bool has1,
+                                          const EpiOperands& o) {
+    if constexpr (EPI == EPI_STORE) {
+        float* out = p.out + static_cast<size_t>(b) * p.out_stride;
+        out[row] = v0 + o.b0;
+        if (has1) out[row + 1] = v1 + o.b1;
+        if (p.advance && b == 0 && row == 0) p.advance->pos += 1;
+    } else if constexpr (EPI == EPI_RESID) {
+        // y += b, then y += x @ W (inference.cpp:22-28)
+        float* out = p.out + static_cast<size_t>(b) * p.out_stride;
+        out[row] = (o.r0 + o.b0) + v0;
+        if (has1) out[row + 1] = (o.r1 + o.b1) + v1;
+    } else if constexpr (EPI == EPI_GELU) {
+        float* out = p.out + static_cast<size_t>(b) * p.out_stride;
+        out[row] = gelu_tanh(v0 + o.b0);
+        if (has1) out[row + 1] = gelu_tanh(v1 + o.b1);
+    } else if constexpr (EPI == EPI_SWIGLU) {
+        // rows (2p, 2p+1) = (gate_p, up_p): hidden_p = up * silu(gate) (inference.cpp:234-239)
+        p.out[static_cast<size_t>(b) * p.out_stride + (row >> 1)] = v1 * silu(v0);
+    } else if constexpr (EPI == EPI_QKV) {
+        float a = v0 + o.b0;
+        float c = has1 ? v1 + o.b1 : 0.0f;
+        if (p.rope && row < 2 * p.d_model) {
+            const float ra = a * o.cs - c * o.sn;
+            const float rc = a * o.sn + c * o.cs;
+            a = ra;
+            c = rc;
+        }
+        store_qkv(p, b, row, a, o);
+        if (has1) store_qkv(p, b, row + 1, c, o);
     }
 }
 
 template <int EPI>
 __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, int b, int row, float v0,
                                               float v1, bool has1) {
-    if constexpr (EPI == EPI_STORE) {
-        float* o = p.out + static_cast<size_t>(b) * p.out_stride;
-        o[row] = v0 + (p.bias ? p.bias[row] : 0.0f);
-        if (has1) o[row + 1] = v1 + (p.bias ? p.bias[row + 1] : 0.0f);
-        if (p.advance && b == 0 && row == 0) p.advance->pos += 1;
-    } else if constexpr (EPI == EPI_RESID) {
-        // y += b, then y += x @ W (inference.cpp:22-28)
-        float* o = p.out + static_cast<size_t>(b) * p.out_stride;
-        o[row] = (o[row] + (p.bias ? p.bias[row] : 0.0f)) + v0;
-        if (has1) o[row + 1] = (o[row + 1] + (p.bias ? p.bias[row + 1] : 0.0f)) + v1;
-    } else if constexpr (EPI == EPI_GELU) {
-        float* o = p.out + static_cast<size_t>(b) * p.out_stride;
-        o[row] = gelu_tanh(v0 + p.bias[row]);
-        if (has1) o[row + 1] = gelu_tanh(v1 + p.bias[row + 1]);
-    } else if constexpr (EPI == EPI_SWIGLU) {
-        // rows (2p, 2p+1) = (gate_p, up_p): hidden_p = up * silu(gate) (inference.cpp:234-239)
-        p.out[static_cast<size_t>(b) * p.out_stride + (row >> 1)] = v1 * silu(v0);
-    } else if constexpr (EPI == EPI_QKV) {
-        int pos, seq = b;
-        if (p.rows_per_seq > 0) {
-            seq = b / p.rows_per_seq;
-            pos = p.pos_base + (b - seq * p.rows_per_seq);
-        } else {
-            pos = p.st->pos;
-        }
-        float a = v0 + p.bias[row];
-        float c = has1 ? v1 + p.bias[row + 1] : 0.0f;
-        if (p.rope && row < 2 * p.d_model) {
-            // head_size is even under RoPE, so (row, row+1) is one rotation pair.
-            const int hs = p.kv.head_size;
-            const int j = ((row % p.d_model) % hs) >> 1;
-            const float cs = p.rope_cos[pos * (hs >> 1) + j];
-            const float sn = p.rope_sin[pos * (hs >> 1) + j];
-            const float ra = a * cs - c * sn;
-            const float rc = a * sn + c * cs;
-            a = ra;
-            c = rc;
-        }
-        store_qkv(p, b, seq, row, a, pos);
-        if (has1) store_qkv(p, b, seq, row + 1, c, pos);
-    }
+    epi_apply<EPI>(p, b, row, v0, v1, has1, epi_fetch<EPI>(p, b, row, has1));
 }
 
 // Normalises a register-resident row slice in place (layer_norm_row,
