@@ -206,6 +206,14 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
     const int K = p.K;
     const float* xin = p.in + static_cast<size_t>(b) * p.in_stride;
     float acc[R];
+    // what the epilogue reads is requested before the products (every lane asks
+    // for the same addresses; lane 0 uses them)
+    EpiOperands epi[PAIRS];
+#pragma unroll
+    for (int q = 0; q < PAIRS; q++) {
+        const int row = row0 + 2 * q;
+        if (row < p.N) epi[q] = epi_fetch<EPI>(p, b, row, row + 1 < p.N);
+    }
 
     if constexpr (KV > 0) {
         // Weight loads are issued first: they do not depend on the activations.
@@ -264,7 +272,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
 #pragma unroll
         for (int q = 0; q < PAIRS; q++) {
             const int row = row0 + 2 * q;
-            if (row < p.N) gemv_epilogue<EPI>(p, b, row, acc[2 * q], acc[2 * q + 1], row + 1 < p.N);
+            if (row < p.N) epi_apply<EPI>(p, b, row, acc[2 * q], acc[2 * q + 1], row + 1 < p.N, epi[q]);
         }
     }
 }
