@@ -169,3 +169,32 @@ def test_eval_scores_a_token_file(setup, tmp_path):
     out = subprocess.run([exe, str(d / "m.bin"), str(other), "--seq", str(seq)], capture_output=True, text=True)
     assert out.returncode == 1 and "token files and checkpoint disagree on vocab size" in out.stderr
     assert subprocess.run([exe, str(d / "m.bin")], capture_output=True).returncode == 2
+
+
+def test_generate_with_a_v1_tokenizer_cache(tmp_path):
+    """A checkpoint trained with the v1 whitespace BPE (the reference's default for checkpoints
+    that record no tokenizer, src/cli/common.cpp:160-187): same command, the cache file in
+    place of the GTOK file."""
+    v1 = R.train_v1(TEXT.replace("\n", " ").encode() * 3, 140)
+    (tmp_path / "v1.cache").write_bytes(v1.cache_image())
+    cfg = synth.Config(synth.ARCH_GPT2, v1.vocab_size, 128, 2, 2, 64)
+    W = synth.make_weights(cfg, 33, std=lively_std(cfg), norm_noise=0.1)
+    synth.write_checkpoint(str(tmp_path / "m.bin"), cfg, W, fingerprint=(1, v1.fingerprint()))
+    om = O.Model.from_tensors(cfg, W)
+    prompt = "Once upon a time,  the little cat"
+    out = run(tmp_path / "m.bin", tmp_path / "v1.cache", prompt, "--max-tokens", 10, "--repetition-penalty", 1.2,
+              "--greedy")
+    assert out.returncode == 0, out.stdout + out.stderr
+    ids = v1.encode(prompt.encode())
+    greedy = O.generate_greedy(om, ids, 10, 1.2)
+    assert f"Tokenizer: {tmp_path / 'v1.cache'} (v1, vocab {v1.vocab_size})\n".encode() in out.stdout
+    assert b"--- Greedy Decoding ---\n\n" + f'Prompt: "{prompt}"\n'.encode() + v1.decode(greedy) + b"\n" in out.stdout
+    # the same checkpoint refuses another v1 vocabulary of the same size
+    vocab = sorted(v1.vocab.items(), key=lambda kv: kv[1])
+    other = R.BpeV1Ref(vocab[:-1] + [(b"\x7f\x7f", vocab[-1][1])], v1.merges[:-1])
+    assert other.vocab_size == v1.vocab_size and other.fingerprint() != v1.fingerprint()
+    (tmp_path / "other.cache").write_bytes(other.cache_image())
+    out = run(tmp_path / "m.bin", tmp_path / "other.cache", prompt, "--greedy")
+    assert out.returncode == 1
+    assert (f"Error: tokenizer v1:{other.fingerprint():016x} is not the one {tmp_path / 'm.bin'} was trained with "
+            f"(v1:{v1.fingerprint():016x})").encode() in out.stderr
