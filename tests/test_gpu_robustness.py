@@ -101,3 +101,31 @@ def test_sessions_and_models_give_their_memory_back(llama768):
         cycle()
     free1 = free_bytes()
     assert free0 - free1 < 8 << 20, f"{(free0 - free1) >> 20} MiB not returned after 10 create/free cycles"
+
+
+def test_prompt_longer_than_one_pass_slice():
+    """More prompt rows than one pass takes at a time (32768): the pass runs in slices of
+    positions, each attending to the cache rows of the slices before it."""
+    cfg = synth.Config(synth.ARCH_MODERN, 301, 128, 1, 2, 1024)
+    W = synth.make_weights(cfg, 17, std=lively_std(cfg), norm_noise=0.1)
+    om, gm = O.Model.from_tensors(cfg, W), G.Model.from_tensors(cfg, W)
+    B, n = 40, 900   # 36000 rows: slices of 819 and 81 positions
+    tokens = synth.uniform_tokens(B * (n + 1), cfg.vocab, 18).reshape(B, n + 1)
+    ids = np.ascontiguousarray(tokens[:, :-1])
+    one_pass = G.Session(gm, batch=B)
+    last = one_pass.prefill(ids)
+    stepwise = G.Session(gm, batch=B, flags=G.FLAG_STEPWISE_PROMPT)
+    want = stepwise.prefill(ids)
+    for b in range(B):
+        assert_logits_close(last[b], want[b], 2e-5, f"sequence {b}")
+    for pos in (0, 818, 819, 899):   # either side of the slice boundary
+        for kv in (0, 1):
+            assert np.abs(one_pass.read_kv(B - 1, 0, kv, pos) - stepwise.read_kv(B - 1, 0, kv, pos)).max() <= 1e-5
+    # one sequence against the CPU oracle, and the scored form of the same pass
+    s = O.Session(om)
+    for t in ids[7]:
+        ref = s.step(int(t))
+    assert_logits_close(last[7], ref, 1e-4, "oracle, sequence 7")
+    nll = G.Session(gm, batch=B).score(ids, tokens[:, 1:])
+    ref_nll = O.score(om, ids[7], tokens[7, 1:])
+    assert np.abs(nll[7] - ref_nll).max() <= 2e-4 * max(1.0, np.abs(ref_nll).max())
