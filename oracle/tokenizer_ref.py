@@ -11,8 +11,10 @@ What it follows and what pins it:
   class "other" each, as pretokenize.cpp:53-90 treats them.  Pinned by the golden
   splits of tests/unit/test_tokenizer.cpp:184-241 (tests/golden/tokenizer_cases.json).
   The `regex` module carries its own Unicode database (17.0 with regex 2026.7.19);
-  grad.cpp's tables are Unicode 16.0.0: code points first assigned after 16.0
-  are "parity unpinned".
+  grad.cpp's tables are Unicode 16.0.0, so the letters and digits that 17.0 added
+  (AGE_17, from the standard's DerivedAge data) are taken out of \p{L} and \p{N}
+  here; the endpoints of those ranges are pinned as class "other" by samples of
+  grad.cpp's own table in tests/golden/tokenizer_cases.json.
 * encode_ordinary(): merges applied in rank order, every occurrence left to right
   (the definition grad.cpp's tests check the fast encoder against,
   tests/unit/test_tokenizer.cpp:150-171).
@@ -34,8 +36,21 @@ from collections import Counter
 
 import regex
 
+# Letters and digits first assigned in Unicode 17.0 (unassigned, hence "other", in 16.0).
+AGE_17 = [
+    (0x088F, 0x088F), (0x0C5C, 0x0C5C), (0x0CDC, 0x0CDC), (0xA7CE, 0xA7CF), (0xA7D2, 0xA7D2), (0xA7D4, 0xA7D4),
+    (0xA7F1, 0xA7F1), (0x10940, 0x10959), (0x10EC5, 0x10EC7), (0x11DB0, 0x11DDB), (0x11DE0, 0x11DE9),
+    (0x16EA0, 0x16EB8), (0x16EBB, 0x16ED3), (0x16FF2, 0x16FF6), (0x187F8, 0x187FF), (0x18D09, 0x18D1E),
+    (0x18D80, 0x18DF2), (0x1E6C0, 0x1E6DE), (0x1E6E0, 0x1E6E2), (0x1E6E4, 0x1E6E5), (0x1E6E7, 0x1E6ED),
+    (0x1E6F0, 0x1E6F4), (0x1E6FE, 0x1E6FF), (0x2B73A, 0x2B73F), (0x2CEA2, 0x2CEAD), (0x323B0, 0x33479),
+]
+_NEW = "".join(f"\\U{lo:08X}-\\U{hi:08X}" for lo, hi in AGE_17)
+LETTER_16 = rf"[\p{{L}}--[{_NEW}]]"
+NUMBER_16 = rf"[\p{{N}}--[{_NEW}]]"
+OTHER_16 = rf"[[^\s\p{{L}}\p{{N}}]||[{_NEW}]]"
+# GPT-2's pattern with the classes of Unicode 16.0 ((?V1): set difference and union)
 GPT2_PATTERN = regex.compile(
-    r"""'s|'t|'re|'ve|'m|'ll|'d| ?\p{L}+| ?\p{N}+| ?[^\s\p{L}\p{N}]+|\s+(?!\S)|\s+""")
+    rf"""(?V1)'s|'t|'re|'ve|'m|'ll|'d| ?{LETTER_16}+| ?{NUMBER_16}+| ?{OTHER_16}+|\s+(?!\S)|\s+""")
 EOT = b"<|endoftext|>"
 
 

@@ -74,6 +74,17 @@ CLASSES = [
     (0x2167, NUMBER), (0x0663, NUMBER), (0x1F600, OTHER), (0x10FFFF, OTHER),
 ]
 
+# What grad.cpp's Unicode 16.0.0 class table (src/tokenizer/unicode_tables.h) says at the ends of
+# the ranges that Unicode 17.0 filled with letters and digits: unassigned in 16.0, so "other";
+# and at their assigned neighbours.
+CLASSES += [(cp, OTHER) for cp in (
+    0x088F, 0x0C5C, 0x0CDC, 0xA7CE, 0xA7CF, 0xA7D2, 0xA7D4, 0xA7F1, 0x10940, 0x10959, 0x10EC5, 0x10EC7, 0x11DB0,
+    0x11DDB, 0x11DE0, 0x11DE9, 0x16EA0, 0x16EB8, 0x16EBB, 0x16ED3, 0x16FF2, 0x16FF6, 0x187F8, 0x187FF, 0x18D09,
+    0x18D1E, 0x18D80, 0x18DF2, 0x1E6C0, 0x1E6DE, 0x1E6E0, 0x1E6E2, 0x1E6E4, 0x1E6E5, 0x1E6E7, 0x1E6ED, 0x1E6F0,
+    0x1E6F4, 0x1E6FE, 0x1E6FF, 0x2B73A, 0x2B73F, 0x2CEA2, 0x2CEAD, 0x323B0, 0x33479)]
+CLASSES += [(0x088E, LETTER), (0xA7CD, LETTER), (0xA7D3, LETTER), (0x187F7, LETTER), (0x18D08, LETTER),
+            (0x2B739, LETTER), (0x2CEA1, LETTER), (0x323AF, LETTER), (0x3347A, OTHER), (0x10EC4, LETTER)]
+
 # the first byte of each is one invalid scalar on its own
 INVALID_UTF8 = [b"\xC0\xAF", b"\xE0\x80\xAF", b"\xED\xA0\x80", b"\xF4\x90\x80\x80", b"\xE6\x97", b"\x80", b"\xFF"]
 

@@ -105,13 +105,22 @@ def test_character_classes():
 
 
 def test_every_codepoint_class_matches_the_regex_module():
+    """All 1,114,112 code points against the `regex` module, whose database is newer than the
+    tokenizer's Unicode 16.0: the letters and digits added since are "other" here (their range
+    ends are pinned by samples of grad.cpp's table in test_character_classes)."""
     import regex
     kinds = [regex.compile(p) for p in (r"\p{L}", r"\p{N}", r"\s")]
+    newer = set()
+    for lo, hi in R.AGE_17:
+        newer.update(range(lo, hi + 1))
     lib = G.load_library()
     bad = []
     for cp in range(0x110000):
         ch = chr(cp)
         want = 3 if kinds[2].match(ch) else 1 if kinds[0].match(ch) else 2 if kinds[1].match(ch) else 0
+        if cp in newer:
+            assert want in (1, 2), hex(cp)
+            want = 0
         if lib.gh_codepoint_class(cp) != want:
             bad.append(hex(cp))
     assert not bad, bad[:20]
