@@ -528,7 +528,9 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
 template <class Get>
 __device__ inline float block_ordered_total(Get get, int n, float* parts) {
     const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
-    const int run = (n + nt - 1) / nt;
+    // an odd run length: lane l starts at l * run, and an even stride would put
+    // many lanes of a wavefront on the same LDS bank at every step of the walk
+    const int run = ((n + nt - 1) / nt) | 1;
     const int lo = min(n, tid * run), hi = min(n, lo + run);
     float part = 0.0f;
     run_pass(get, lo, hi, [&](int, float x) {
@@ -550,7 +552,9 @@ __device__ inline float block_ordered_total(Get get, int n, float* parts) {
 template <class Get>
 __device__ inline int block_first_reach(Get get, int n, float thr, float* parts, int* slot) {
     const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6;
-    const int run = (n + nt - 1) / nt;
+    // an odd run length: lane l starts at l * run, and an even stride would put
+    // many lanes of a wavefront on the same LDS bank at every step of the walk
+    const int run = ((n + nt - 1) / nt) | 1;
     const int lo = min(n, tid * run), hi = min(n, lo + run);
     float part = 0.0f;
     run_pass(get, lo, hi, [&](int, float x) {
