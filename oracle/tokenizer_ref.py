@@ -12,7 +12,7 @@ What it follows and what pins it:
   splits of tests/unit/test_tokenizer.cpp:184-241 (tests/golden/tokenizer_cases.json).
   The `regex` module carries its own Unicode database (17.0 with regex 2026.7.19);
   grad.cpp's tables are Unicode 16.0.0, so the letters and digits that 17.0 added
-  (AGE_17, from the standard's DerivedAge data) are taken out of \p{L} and \p{N}
+  (AGE_17, from the standard's DerivedAge data) are taken out of the letter and number classes
   here; the endpoints of those ranges are pinned as class "other" by samples of
   grad.cpp's own table in tests/golden/tokenizer_cases.json.
 * encode_ordinary(): merges applied in rank order, every occurrence left to right
