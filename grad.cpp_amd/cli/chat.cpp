@@ -3,10 +3,12 @@
 // (src/cli/chat.cpp:18-71 of grad.cpp):
 //
 //   gradhip-chat <checkpoint> <tokenizer.tok> [--max-tokens N] [--temperature T] [--top-k K]
-//       [--top-p P] [--repetition-penalty R] [--greedy] [--seed S]
+//       [--top-p P] [--repetition-penalty R] [--greedy] [--seed S] [--stop-at-eos]
 //
 // An empty line, "exit" or "quit" ends the session.  As in the reference, each
 // line starts from an empty context (text_gen.cpp:100) and --greedy means top-k 1.
+// --stop-at-eos (not in grad.cpp, whose replies always run to --max-tokens) ends a
+// reply after the tokenizer's end-of-text token.
 #include "gradhip.hpp"
 #include "options.h"
 
@@ -32,6 +34,7 @@ int main(int argc, char** argv) {
         gradhip::check_tokenizer_matches(model, *tokenizer, o.positional[0]);
         gradhip::TextGen generator(model, tokenizer.get());
         if (o.seed) generator.set_seed(*o.seed);
+        if (o.stop_at_eos) generator.set_stop_token(tokenizer->eos_id());
         const int top_k = o.greedy ? 1 : o.top_k;
 
         std::cout << "\nThis is a base language model: it continues text in the"

@@ -25,6 +25,7 @@ struct Options {
     float repetition_penalty = 1.2f;
     bool greedy = false;
     std::optional<std::uint64_t> seed;
+    bool stop_at_eos = false;  // not in grad.cpp: end a streamed reply at the tokenizer's end-of-text id
 };
 
 template <class T>
@@ -60,6 +61,8 @@ inline Options parse(int argc, char** argv, Options o) {
             if (!(o.repetition_penalty > 0.0f)) throw Usage("--repetition-penalty: must be positive");
         } else if (a == "--greedy") {
             o.greedy = true;
+        } else if (a == "--stop-at-eos") {
+            o.stop_at_eos = true;
         } else if (a == "--seed") {
             o.seed = number<std::uint64_t>(a, value());
         } else if (a.rfind("--", 0) == 0) {

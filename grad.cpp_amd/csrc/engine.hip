@@ -381,6 +381,10 @@ struct Session {
     float* host_logits = nullptr;  // pinned, B * V
     int* host_ids = nullptr;       // pinned staging for ids
     int* host_err = nullptr;       // pinned landing spot for the device error flag
+    // streaming from the persistent kernel: pinned words the kernel writes / reads directly
+    unsigned long long* feed = nullptr;  // [hist_stride] {token, tag} per pick of a launch
+    unsigned* stop_word = nullptr;       // set by the host to end a run at the next pick
+    unsigned feed_base = 0;              // tags of a launch are feed_base + 1 ...; never reused
 
     int pos = 0;     // host mirror of DevState
     int n_hist = 0;
@@ -421,6 +425,8 @@ struct Session {
         if (host_logits) (void)hipHostFree(host_logits);
         if (host_ids) (void)hipHostFree(host_ids);
         if (host_err) (void)hipHostFree(host_err);
+        if (feed) (void)hipHostFree(feed);
+        if (stop_word) (void)hipHostFree(stop_word);
         if (stream) (void)hipStreamDestroy(stream);
     }
 };
@@ -642,21 +648,23 @@ using PersistKernel = void (*)(const PersistParams);
 // The shapes the persistent kernel is built for (head size 64, d_model and FFN
 // width multiples of 256); nullptr for anything else.
 // row_lds: the sampler's working row fits in LDS.
-template <bool ROW_LDS>
+template <bool ROW_LDS, bool FEED>
 static PersistKernel persist_kernel_of(const Shape& sh) {
     if (sh.head_size() != 64) return nullptr;
     const int d = sh.d_model, F = sh.d_ff();
     if (sh.modern()) {
-        if (d == 768 && F == 2048) return persist_decode_kernel<3, 8, true, ROW_LDS>;
+        if (d == 768 && F == 2048) return persist_decode_kernel<3, 8, true, ROW_LDS, FEED>;
         return nullptr;
     }
-    if (d == 512) return persist_decode_kernel<2, 8, false, ROW_LDS>;
-    if (d == 768) return persist_decode_kernel<3, 12, false, ROW_LDS>;
-    if (d == 1024) return persist_decode_kernel<4, 16, false, ROW_LDS>;
+    if (d == 512) return persist_decode_kernel<2, 8, false, ROW_LDS, FEED>;
+    if (d == 768) return persist_decode_kernel<3, 12, false, ROW_LDS, FEED>;
+    if (d == 1024) return persist_decode_kernel<4, 16, false, ROW_LDS, FEED>;
     return nullptr;
 }
-static PersistKernel persist_kernel_for(const Shape& sh, bool row_lds) {
-    return row_lds ? persist_kernel_of<true>(sh) : persist_kernel_of<false>(sh);
+// feed: the variant that reports its picks to the host and can be told to stop.
+static PersistKernel persist_kernel_for(const Shape& sh, bool row_lds, bool feed = false) {
+    if (feed) return row_lds ? persist_kernel_of<true, true>(sh) : persist_kernel_of<false, true>(sh);
+    return row_lds ? persist_kernel_of<true, false>(sh) : persist_kernel_of<false, false>(sh);
 }
 
 static const char* persist_unavailable(const Session& s, int lds_bytes, int cus) {
@@ -670,9 +678,11 @@ static const char* persist_unavailable(const Session& s, int lds_bytes, int cus)
 }
 
 // One launch: n_prompt steps fed from the history, then rounds of pick + step.
+// feed: the kernel reports every pick in the session's pinned feed and honours its
+// stop word and stop_token.
 static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool start_with_pick,
                         const gh_sampling* o, const float* dev_uniforms, int u_stride, uint64_t seed,
-                        float* logit_log) {
+                        float* logit_log, bool feed = false, int stop_token = -1) {
     const Model& m = *s.m;
     const Shape& sh = m.shape;
     if (n_steps <= 0 && n_picks <= 0) return;
@@ -713,6 +723,14 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     p.spin_limit = 1u << 18;
     p.prof = s.prof;
     p.prof_cap = s.prof_cap;
+    p.stop_token = -1;
+    if (feed) {
+        p.feed = s.feed;
+        p.feed_base = s.feed_base;
+        p.stop_request = s.stop_word;
+        p.stop_token = stop_token;
+        s.feed_base += static_cast<unsigned>(n_picks) + 1u;
+    }
     PickParams& k = p.pick;
     k.logits = s.logits;
     k.V = sh.vocab;
@@ -736,7 +754,7 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     k.work_stride = s.work_stride;
     k.sort_cap = kPickWorkFloats;
 
-    PersistKernel kernel = persist_kernel_for(sh, s.pick_row_in_lds);
+    PersistKernel kernel = persist_kernel_for(sh, s.pick_row_in_lds, feed);
     hipLaunchKernelGGL(kernel, dim3(s.persist_grid), dim3(kPersistThreads), s.persist_lds, s.stream, p);
     HIP_CHECK(hipGetLastError());
 
@@ -868,6 +886,10 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     HIP_CHECK(hipHostMalloc(&s.host_logits, B * V * sizeof(float)));
     HIP_CHECK(hipHostMalloc(&s.host_ids, B * s.hist_stride * sizeof(int)));
     HIP_CHECK(hipHostMalloc(&s.host_err, sizeof(int)));
+    HIP_CHECK(hipHostMalloc(&s.feed, s.hist_stride * sizeof(unsigned long long), hipHostMallocCoherent));
+    HIP_CHECK(hipHostMalloc(&s.stop_word, sizeof(unsigned), hipHostMallocCoherent));
+    std::memset(s.feed, 0, s.hist_stride * sizeof(unsigned long long));
+    *s.stop_word = 0;
 
     // Attention chunking: a (sequence, head) is split over several workgroups
     // only while that is needed to cover the GPU (at least ~512 workgroups); a
@@ -915,9 +937,10 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
                 s.prof_cap = 1 << 16;
                 dev_alloc(s.prof, s.prof_cap);
             }
-            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(persist_kernel_for(sh, s.pick_row_in_lds)),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          static_cast<int>(s.persist_lds)));
+            for (const bool feed : {false, true})
+                HIP_CHECK(hipFuncSetAttribute(
+                    reinterpret_cast<const void*>(persist_kernel_for(sh, s.pick_row_in_lds, feed)),
+                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(s.persist_lds)));
             s.launches_per_step = 1;
         }
     }
@@ -1787,6 +1810,104 @@ gh_status gh_session_decode(gh_session* sess, int32_t max_tokens, const gh_sampl
             for (size_t b = 0; b < B; b++)
                 std::memcpy(out_ids + b * max_tokens, s.host_ids + b * s.hist_stride,
                             made * sizeof(int));
+        *out_count = made;
+        HIP_CHECK(hipEventElapsedTime(&s.timing.decode_ms, s.ev[1], s.ev[2]));
+        s.timing.decode_steps = stepped;
+    });
+}
+
+gh_status gh_session_decode_stream(gh_session* sess, int32_t max_tokens, const gh_sampling* opt,
+                                   const float* uniforms, uint64_t seed, int32_t stop_token,
+                                   gh_token_callback on_tokens, void* user, int32_t* out_ids,
+                                   int32_t* out_count) {
+    return guard([&] {
+        if (!sess || !opt || !out_count || !on_tokens) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        Session& s = *sess->impl;
+        check_sampling(*opt);
+        *out_count = 0;
+        s.timing = gh_timing{};
+        s.timing.launches_per_step = s.launches_per_step;
+        if (max_tokens <= 0) return;
+        if (s.pos == 0) throw ApiError{GH_ERR_RUNTIME, "no logits yet: step or prefill first"};
+        const int B = s.B, C = s.m->shape.max_len;
+        const float* du = opt->greedy ? nullptr : stage_uniforms(s, uniforms, static_cast<size_t>(B) * max_tokens);
+        const int saved_picks = s.picks;
+        if (du) s.picks = 0;  // uniforms are indexed from this call's first pick
+        int made = 0, stepped = 0;
+        HIP_CHECK(hipEventRecord(s.ev[1], s.stream));
+        if (s.engine == GH_ENGINE_PERSISTENT) {
+            // One launch runs the whole loop; the kernel reports each pick in pinned
+            // memory as it is made and this thread hands it on while the kernel goes on.
+            int planned_picks = 0, planned_steps = 0, pos = s.pos, nh = s.n_hist;
+            for (int i = 0; i < max_tokens; i++) {
+                if (nh >= s.hist_stride) break;
+                planned_picks++;
+                nh++;
+                if (pos >= C) break;
+                planned_steps++;
+                pos++;
+            }
+            __atomic_store_n(s.stop_word, 0u, __ATOMIC_RELEASE);
+            const unsigned base = s.feed_base;
+            persist_run(s, 0, planned_steps, planned_picks, true, opt, du, max_tokens, seed, nullptr, true,
+                        stop_token);
+            HIP_CHECK(hipEventRecord(s.ev[2], s.stream));
+            bool kernel_done = false;
+            unsigned idle = 0;
+            while (made < planned_picks) {
+                const unsigned long long w = __atomic_load_n(s.feed + made, __ATOMIC_ACQUIRE);
+                if (static_cast<unsigned>(w >> 32) == base + static_cast<unsigned>(made) + 1u) {
+                    const int32_t tok = static_cast<int32_t>(static_cast<unsigned>(w));
+                    if (tok < 0) break;  // the kernel saw the stop word before this pick
+                    if (out_ids) out_ids[made] = tok;
+                    const int32_t asked = on_tokens(user, &tok, made);
+                    made++;
+                    idle = 0;
+                    if (asked != 0) __atomic_store_n(s.stop_word, 1u, __ATOMIC_RELEASE);
+                    if (tok == stop_token) break;  // the kernel ends after this token's step
+                    continue;
+                }
+                if (kernel_done) break;  // the launch is over and reported no further pick
+                if ((++idle & 255u) == 0u) {
+                    const hipError_t q = hipStreamQuery(s.stream);
+                    if (q == hipSuccess) kernel_done = true;  // read the feed once more, then leave
+                    else if (q != hipErrorNotReady) HIP_CHECK(q);
+                }
+            }
+            HIP_CHECK(hipStreamSynchronize(s.stream));
+            check_persist_abort(s);
+            // persist_run advanced the host's view by the planned run: take back what was not run
+            stepped = std::min(made, planned_steps);
+            s.pos -= planned_steps - stepped;
+            s.arrive_total -= static_cast<unsigned>(planned_steps - stepped);
+            s.n_hist -= planned_picks - made;
+            s.picks -= planned_picks - made;
+        } else {
+            std::vector<char> seen(static_cast<size_t>(B), 0);
+            int n_seen = 0;
+            for (int i = 0; i < max_tokens; i++) {
+                if (s.n_hist >= s.hist_stride) break;
+                launch_pick(s, *opt, du, max_tokens, seed, true);
+                HIP_CHECK(hipMemcpyAsync(s.host_ids, s.tok, B * sizeof(int), hipMemcpyDeviceToHost, s.stream));
+                HIP_CHECK(hipStreamSynchronize(s.stream));
+                if (out_ids)
+                    for (int b = 0; b < B; b++) out_ids[static_cast<size_t>(b) * max_tokens + i] = s.host_ids[b];
+                const int32_t asked = on_tokens(user, s.host_ids, i);
+                made++;
+                for (int b = 0; b < B; b++)
+                    if (s.host_ids[b] == stop_token && !seen[b]) {
+                        seen[b] = 1;
+                        n_seen++;
+                    }
+                if (s.pos >= C) break;
+                run_step(s);
+                stepped++;
+                if (asked != 0 || n_seen == B) break;
+            }
+            HIP_CHECK(hipEventRecord(s.ev[2], s.stream));
+            HIP_CHECK(hipStreamSynchronize(s.stream));
+        }
+        if (du) s.picks = saved_picks + made;
         *out_count = made;
         HIP_CHECK(hipEventElapsedTime(&s.timing.decode_ms, s.ev[1], s.ev[2]));
         s.timing.decode_steps = stepped;

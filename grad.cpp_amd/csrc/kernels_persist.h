@@ -64,6 +64,16 @@ struct PersistParams {
     unsigned arrive_base;  // logits phases completed before this launch
     PickParams pick;
     unsigned spin_limit;
+    // Streaming (all optional).  feed: pinned host memory, one 8-byte {token, tag}
+    // word per pick of this launch, tag = feed_base + pick number + 1, written as
+    // each token is picked so the host can hand it on while the kernel goes on; a
+    // token of -1 says the run ended before that pick.  stop_request: a pinned host
+    // word the host sets to end the run at the next pick.  stop_token: the run ends
+    // after the step that follows a pick of this token (-1: none).
+    unsigned long long* feed;
+    unsigned feed_base;
+    const unsigned* stop_request;
+    int stop_token;
     unsigned long long* prof;  // optional: phase-end timestamps of workgroup 0 (100 MHz clock)
     int prof_cap;
 };
@@ -124,11 +134,19 @@ __device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float*
     return true;
 }
 
+// Reports pick number i_pick of this launch to the host: one 8-byte word in pinned memory.
+__device__ __forceinline__ void feed_put(const PersistParams& p, int i_pick, int token) {
+    const unsigned long long w =
+        (static_cast<unsigned long long>(p.feed_base + static_cast<unsigned>(i_pick) + 1u) << 32)
+        | static_cast<unsigned long long>(static_cast<unsigned>(token));
+    __hip_atomic_store(p.feed + i_pick, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // One pick by workgroup 0 (text_gen.cpp:48-61 / :80-86): waits until every
 // workgroup's logits rows have landed, picks, records the token in the history
 // and publishes it in the token cell.  The other workgroups return at once and
 // learn the token from the cell.  False: the wait was abandoned.
-template <bool ROW_LDS>
+template <bool ROW_LDS, bool FEED>
 __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds, int i_pick,
                                     unsigned arrive_gen, unsigned tok_tag, bool wait_logits) {
     if (blockIdx.x != 0) return true;
@@ -139,6 +157,18 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
     pk.pick_idx = p.pick.pick_idx + i_pick;
     // the draw needs no logits: form it while they arrive
     const float u = pk.greedy ? 0.0f : pick_draw(pk, 0);
+    // The host's stop request (one trip over the bus while the other workgroups'
+    // logits arrive): no pick; every workgroup leaves when it reads the token cell.
+    if constexpr (FEED) {
+        const unsigned stop = __hip_atomic_load(p.stop_request, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (__builtin_amdgcn_readfirstlane(stop) != 0u) {
+            if (tid == 0) {
+                cell_put(p.tokc, __int_as_float(-1), tok_tag);
+                feed_put(p, i_pick, -1);
+            }
+            return false;
+        }
+    }
     if (wait_logits) {
         // one wavefront watches the 16 arrival counters; the workgroup meets once
         bool failed = false;
@@ -176,6 +206,7 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
     if (tid == 0) {
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         cell_put(p.tokc, __int_as_float(chosen), tok_tag);
+        if constexpr (FEED) feed_put(p, i_pick, chosen);
         if (pp) pp[1] = __builtin_amdgcn_s_memrealtime();
     }
     return true;
@@ -289,8 +320,9 @@ __device__ __forceinline__ void load_qkv_operands(const PersistParams& p, const 
     }
 }
 
-// KD = d_model / 256, KF = FFN width / 256; head size 64.
-template <int KD, int KF, bool MODERN, bool ROW_LDS>
+// KD = d_model / 256, KF = FFN width / 256; head size 64.  FEED: the streaming
+// variant (feed, stop word, stop token); the plain one carries none of it.
+template <int KD, int KF, bool MODERN, bool ROW_LDS, bool FEED>
 __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const PersistParams p) {
     extern __shared__ __attribute__((aligned(128))) float lds[];
     constexpr int D = KD * 256, F = KF * 256, HS = 64;
@@ -309,6 +341,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     int i_pick = 0;
     unsigned arrive_gen = p.arrive_base;
     int n_stamp = 0;
+    bool ended = false;  // a picked token was the stop token
     auto stamp = [&]() {
         if (p.prof && wg == 0 && tid == 0 && n_stamp < p.prof_cap) p.prof[n_stamp] = __builtin_amdgcn_s_memrealtime();
         n_stamp++;
@@ -332,10 +365,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         // ===== pick before step s (text_gen.cpp:48-61): the first one of a launch may
         // use logits that are already in memory, later ones follow step s - 1.  One call
         // site: the sampler is the largest piece of code in the kernel.
-        if (i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick)) {
+        if ((!FEED || !ended) && i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick)) {
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
-            if (!persist_pick<ROW_LDS>(p, lds, i_pick, arrive_gen, tt, s > 0)) return;
+            if (!persist_pick<ROW_LDS, FEED>(p, lds, i_pick, arrive_gen, tt, s > 0)) return;
             i_pick++;
             if (wg == 0) {
                 // the pick used the whole LDS; restore the page table
@@ -345,7 +378,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             }
         }
         stamp();
-        if (s >= p.n_steps) break;
+        if ((FEED && ended) || s >= p.n_steps) break;
         asm volatile("" : "+v"(tid));  // as in the layer loop below
         wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         lane = tid & 63;
@@ -376,6 +409,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             if (!gather_cells(p.tokc, 1, tt, ascr, p)) return;
             tok = __float_as_int(ascr[0]);
             __syncthreads();
+            if constexpr (FEED) {
+                if (tok < 0) return;          // the host asked for the run to end here
+                ended = tok == p.stop_token;  // this step is the last one
+            }
         }
         for (int j = tid; j < D; j += kPersistThreads) {
             float v = p.E[static_cast<size_t>(tok) * D + j];

@@ -59,6 +59,7 @@ class GhTokenizerInfo(C.Structure):
 
 # Every symbol include/gradhip.h declares: name -> (restype, argtypes)
 _f32p, _i32p, _vp = C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_void_p
+TokenCallback = C.CFUNCTYPE(C.c_int32, C.c_void_p, C.POINTER(C.c_int32), C.c_int32)  # gh_token_callback
 SYMBOLS = {
     "gh_last_error": (C.c_char_p, []),
     "gh_model_load": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
@@ -82,6 +83,8 @@ SYMBOLS = {
     "gh_session_read_kv": (C.c_int, [_vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, _f32p]),
     "gh_session_pick": (C.c_int, [_vp, C.POINTER(GhSampling), _f32p, C.c_uint64, _i32p]),
     "gh_session_decode": (C.c_int, [_vp, C.c_int32, C.POINTER(GhSampling), _f32p, C.c_uint64, _i32p, _i32p]),
+    "gh_session_decode_stream": (C.c_int, [_vp, C.c_int32, C.POINTER(GhSampling), _f32p, C.c_uint64, C.c_int32,
+                                           TokenCallback, _vp, _i32p, _i32p]),
     "gh_session_generate": (C.c_int, [_vp, _i32p, C.c_int32, C.c_int32, C.POINTER(GhSampling), _f32p,
                                       C.c_uint64, _i32p, _i32p, _f32p, _i32p]),
     "gh_session_last_timing": (C.c_int, [_vp, C.POINTER(GhTiming)]),
@@ -376,6 +379,33 @@ class Session:
         _check(load_library().gh_session_decode(
             self._h, max_tokens, C.byref(opt), u.ctypes.data_as(_f32p) if u is not None else None, seed,
             out.ctypes.data_as(_i32p), C.byref(n)))
+        return out[:, :n.value].copy()
+
+    def decode_stream(self, max_tokens, opt: GhSampling, on_tokens, stop_token=-1, uniforms=None, seed=0):
+        """decode() with every round's picks handed to on_tokens(ids, index) as they are made; a
+        true return value asks for the run to end, stop_token ends it after the round that picks
+        it.  Returns the picks (batch, n)."""
+        out = np.zeros((self.batch, max(max_tokens, 1)), dtype=np.int32)
+        n = C.c_int32()
+        u = None
+        if uniforms is not None:
+            u = np.ascontiguousarray(uniforms, dtype=np.float32).reshape(self.batch, max_tokens)
+        failure = []
+
+        def relay(_user, ids, index):
+            if failure:
+                return 1
+            try:
+                return 1 if on_tokens([ids[b] for b in range(self.batch)], index) else 0
+            except BaseException as e:  # raised again once the run has ended
+                failure.append(e)
+                return 1
+
+        _check(load_library().gh_session_decode_stream(
+            self._h, max_tokens, C.byref(opt), u.ctypes.data_as(_f32p) if u is not None else None, seed,
+            stop_token, TokenCallback(relay), None, out.ctypes.data_as(_i32p), C.byref(n)))
+        if failure:
+            raise failure[0]
         return out[:, :n.value].copy()
 
     def generate(self, prompts, max_tokens, opt: GhSampling, uniforms=None, seed=0, want_logits=False):

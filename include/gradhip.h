@@ -184,6 +184,31 @@ gh_status gh_session_decode(gh_session* s, int32_t max_tokens, const gh_sampling
                             const float* uniforms, uint64_t seed, int32_t* out_ids,
                             int32_t* out_count);
 
+/* Receives the picks of one round (ids[b] for sequence b; index counts rounds
+ * from 0) as soon as they exist.  A nonzero return asks for the run to end. */
+typedef int32_t (*gh_token_callback)(void* user, const int32_t* ids, int32_t index);
+
+/* TextGen::generate_stream's loop (text_gen.cpp:107-118) continued from the
+ * session's current context: gh_session_decode with every round's picks handed
+ * to on_tokens as they are made, plus two ways to end before max_tokens, which
+ * the reference lacks (its loop always runs to max_tokens or capacity):
+ *   stop_token >= 0: the run ends once every sequence has picked that id (an
+ *     end-of-text id); the round that picked it is completed (pushed and stepped);
+ *   on_tokens returns nonzero: the run ends as soon as the device learns of it.
+ * With one sequence on the persistent engine the whole loop is ONE kernel launch
+ * that writes each pick to pinned host memory while it goes on computing, and the
+ * calling thread runs on_tokens beside it: a request to stop takes effect a round
+ * or two later, and those rounds' picks are still delivered.  Every round that is
+ * delivered is complete, so *out_count rounds later the session is exactly where
+ * gh_session_decode with max_tokens = *out_count would have left it, and a later
+ * call continues the same stream of picks.  on_tokens must not call into this
+ * session.  out_ids (batch x max_tokens, may be NULL), uniforms and seed as in
+ * gh_session_decode. */
+gh_status gh_session_decode_stream(gh_session* s, int32_t max_tokens, const gh_sampling* opt,
+                                   const float* uniforms, uint64_t seed, int32_t stop_token,
+                                   gh_token_callback on_tokens, void* user, int32_t* out_ids,
+                                   int32_t* out_count);
+
 /* TextGen::generate_greedy / generate_sample (text_gen.cpp:37-91) for `batch`
  * prompts of equal length, with the token loop kept on the GPU.  prompts is
  * batch x prompt_len; out_tokens is batch x (prompt_len + max_tokens) and

@@ -19,6 +19,7 @@
 
 #include <cstdint>
 #include <cstdio>
+#include <exception>
 #include <functional>
 #include <memory>
 #include <optional>
@@ -365,7 +366,8 @@ public:
     }
 
     // Invokes on_text with each token's text as soon as it is sampled; returns
-    // the number of tokens generated (text_gen.cpp:93-120).
+    // the number of tokens generated (text_gen.cpp:93-120).  The loop runs on the
+    // GPU in one launch where the engine allows; on_text runs beside it.
     int generate_stream(const std::vector<int>& prompt_tokens,
                         const std::function<void(const std::string&)>& on_text, float temperature = 1.0f,
                         int max_tokens = 50, float repetition_penalty = 1.2f, int top_k = 0,
@@ -375,21 +377,32 @@ public:
         std::vector<int32_t> ids(prompt_tokens.begin(), prompt_tokens.end());
         check(gh_session_prefill(session.handle(), ids.data(), static_cast<int32_t>(ids.size()), nullptr));
         gh_sampling o{temperature, top_k, top_p, repetition_penalty, 0};
-        const std::uint64_t seed = next_seed();
-        int generated = 0;
-        for (int i = 0; i < max_tokens; i++) {
-            // a pick made with the context already full is pushed but not stepped,
-            // and ends the loop (text_gen.cpp:116)
-            const bool full = session.position() >= session.capacity();
-            int32_t tok = 0, made = 0;
-            check(gh_session_decode(session.handle(), 1, &o, nullptr, seed, &tok, &made));
-            if (made == 0) break;
-            generated++;
-            on_text(tokens_to_string({static_cast<int>(tok)}));
-            if (full) break;
-        }
+        struct Relay {
+            TextGen* self;
+            const std::function<void(const std::string&)>* on_text;
+            std::exception_ptr error;
+        } relay{this, &on_text, nullptr};
+        const gh_token_callback hand_on = [](void* user, const int32_t* picked, int32_t) -> int32_t {
+            Relay& r = *static_cast<Relay*>(user);
+            if (r.error) return 1;
+            try {
+                (*r.on_text)(r.self->tokens_to_string({static_cast<int>(picked[0])}));
+                return 0;
+            } catch (...) {
+                r.error = std::current_exception();  // rethrown once the run has ended
+                return 1;
+            }
+        };
+        int32_t generated = 0;
+        check(gh_session_decode_stream(session.handle(), max_tokens, &o, nullptr, next_seed(), stop_token_, hand_on,
+                                       &relay, nullptr, &generated));
+        if (relay.error) std::rethrow_exception(relay.error);
         return generated;
     }
+
+    // Not in grad.cpp, whose loops always run to max_tokens or capacity:
+    // generate_stream ends after the round that picks this id (an end-of-text id).
+    void set_stop_token(std::optional<int> id) { stop_token_ = id ? *id : -1; }
 
     // The token ids of the last generate_greedy / generate_sample call.
     const std::vector<int>& last_tokens() const { return last_; }
@@ -427,6 +440,7 @@ private:
     const Tokenizer* tokenizer_;
     std::optional<std::uint64_t> seed_;
     std::vector<int> last_;
+    int stop_token_ = -1;
 };
 
 }  // namespace gradhip

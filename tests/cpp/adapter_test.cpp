@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <iostream>
 #include <sstream>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -57,8 +58,31 @@ int main(int argc, char** argv) {
         std::printf("greedy %s\n", gen.generate_greedy(prompt, 12, 1.2f).c_str());
         std::printf("sample %s\n", gen.generate_sample(prompt, 0.8f, 12, 1.1f, 5, 0.9f).c_str());
         std::string streamed;
-        const int n = gen.generate_stream(prompt, [&](const std::string& t) { streamed += t; }, 0.8f, 12, 1.1f, 5, 0.9f);
+        std::vector<int> streamed_ids;
+        const int n = gen.generate_stream(prompt, [&](const std::string& t) {
+            streamed += t;
+            streamed_ids.push_back(std::atoi(t.c_str()));
+        }, 0.8f, 12, 1.1f, 5, 0.9f);
         std::printf("stream %d %s\n", n, streamed.c_str());
+        // what the callback throws reaches the caller, with its type, once the run has ended
+        try {
+            int calls = 0;
+            (void)gen.generate_stream(prompt, [&](const std::string&) {
+                if (++calls == 3) throw std::domain_error("third token");
+            }, 0.8f, 12, 1.1f, 5, 0.9f);
+            std::printf("callback_error none\n");
+        } catch (const std::domain_error& e) {
+            std::printf("callback_error %s\n", e.what());
+        }
+        // a stop token (not in grad.cpp): the stream ends after the first time it is picked
+        {
+            gradhip::TextGen stopper(model, &tok);
+            stopper.set_seed(77);
+            stopper.set_stop_token(streamed_ids.at(4));
+            std::string cut;
+            const int m = stopper.generate_stream(prompt, [&](const std::string& t) { cut += t; }, 0.8f, 12, 1.1f, 5, 0.9f);
+            std::printf("stopped %d %s\n", m, cut.c_str());
+        }
         std::printf("empty [%s]\n", gen.generate_greedy({}, 5).c_str());
         // capacity rule: asks for more tokens than the context can take
         std::printf("overflow %s\n", gen.generate_greedy(prompt, model.getMaxLen() + 10, 1.0f).c_str());

@@ -58,6 +58,11 @@ def test_cpp_caller_matches_the_oracle(tmp_path, arch):
     assert [int(x) for x in lines["sample"].split()] == sampled.tolist()
     st = lines["stream"].split()
     assert int(st[0]) == 12 and [int(x) for x in st[1:]] == sampled.tolist()[len(prompt):]
+    assert lines["callback_error"] == "third token"
+    tail = sampled.tolist()[len(prompt):]
+    cut = tail[:tail.index(tail[4]) + 1]  # ends after the first pick of the stop token
+    sp = lines["stopped"].split()
+    assert int(sp[0]) == len(cut) and [int(x) for x in sp[1:]] == cut
     assert lines["empty"] == "[]"
     over = O.generate_greedy(om, prompt, cfg.max_len + 10, 1.0)
     assert len(over) == cfg.max_len + 1  # the pick after the last step is pushed, then the loop stops

@@ -126,6 +126,16 @@ def test_chat_streams_each_line(setup):
     ids = tok.encode(b"the cat\n")
     greedy = O.generate_greedy(om, ids, 6, 1.0)
     assert out.returncode == 0 and b"> the cat" + tok.decode(greedy[len(ids):]) + b"\n\n> " in out.stdout
+    # --stop-at-eos: the reply ends after the tokenizer's end-of-text id; the stream up to there is
+    # the reference's (which has no stop condition and runs on)
+    eos = tok.vocab_size - 1  # the one special token comes last
+    out = subprocess.run([exe, str(d / "m.bin"), str(d / "t.tok"), "--max-tokens", "40", "--temperature", "1.5",
+                          "--seed", "61", "--stop-at-eos"], input=b"a dog\n\n", capture_output=True, timeout=120)
+    ids = tok.encode(b"a dog\n")
+    ref = list(O.generate_sample(om, ids, synth.uniforms(40, 61), 1.5, 40, 1.2, 0, 1.0)[len(ids):])
+    assert eos in ref[3:30]  # the seed was chosen for this
+    ref = ref[:ref.index(eos) + 1]
+    assert out.returncode == 0 and b"> a dog" + tok.decode(ref) + b"\n\n> " in out.stdout
 
 
 def test_eval_scores_a_token_file(setup, tmp_path):
