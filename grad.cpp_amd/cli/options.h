@@ -25,7 +25,8 @@ struct Options {
     float repetition_penalty = 1.2f;
     bool greedy = false;
     std::optional<std::uint64_t> seed;
-    bool stop_at_eos = false;  // not in grad.cpp: end a streamed reply at the tokenizer's end-of-text id
+    bool stop_at_eos = false;   // not in grad.cpp: end a streamed reply at the tokenizer's end-of-text id
+    bool keep_context = false;  // not in grad.cpp: chat lines continue one live context
 };
 
 template <class T>
@@ -63,6 +64,8 @@ inline Options parse(int argc, char** argv, Options o) {
             o.greedy = true;
         } else if (a == "--stop-at-eos") {
             o.stop_at_eos = true;
+        } else if (a == "--keep-context") {
+            o.keep_context = true;
         } else if (a == "--seed") {
             o.seed = number<std::uint64_t>(a, value());
         } else if (a.rfind("--", 0) == 0) {

@@ -138,6 +138,35 @@ def test_chat_streams_each_line(setup):
     assert out.returncode == 0 and b"> a dog" + tok.decode(ref) + b"\n\n> " in out.stdout
 
 
+def test_chat_can_keep_its_context(setup):
+    """--keep-context (not in grad.cpp, which starts every line from an empty context): a line is
+    appended to the conversation so far, the draws go on where the last reply stopped, and a
+    conversation that no longer fits starts over."""
+    d, tok, cfg, om = setup
+    exe = os.path.join(ROOT, "grad.cpp_amd", "bin", "gradhip-chat")
+    lines = ["the little cat", "sat on", "the mat and the hat"]
+    n = 25
+    out = subprocess.run([exe, str(d / "m.bin"), str(d / "t.tok"), "--max-tokens", str(n), "--temperature", "0.9",
+                          "--top-k", "8", "--repetition-penalty", "1.15", "--seed", "5", "--keep-context"],
+                         input=("\n".join(lines) + "\n\n").encode(), capture_output=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    seed, drawn = 5, 0
+    context, want, started_over = [], b"", 0
+    for line in lines:
+        ids = [int(t) for t in tok.encode((line + "\n").encode())]
+        want += b"> " + line.encode()
+        if len(context) + len(ids) >= cfg.max_len:
+            want += b"\n[context full: starting over]"
+            context, seed, drawn = [], seed + 1, 0  # a fresh session counts its draws from zero
+            started_over += 1
+        ref = O.generate_sample(om, context + ids, synth.uniforms(drawn + n, seed)[drawn:], 0.9, n, 1.15, 8, 1.0)
+        want += tok.decode(ref[len(context) + len(ids):]) + b"\n\n"
+        context = [int(t) for t in ref]
+        drawn += n
+    assert started_over == 1  # the third line does not fit the 64-token context
+    assert out.stdout.endswith(want + b"> ")
+
+
 def test_eval_scores_a_token_file(setup, tmp_path):
     """gradhip-eval: windows of a TOK1 file (src/data/token_file.cpp:149-176) in batches of eight,
     loss as training::mean_loss forms it (src/training/trainer.cpp:319-340)."""
