@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # (32-token prompt already cached): FETCH_SIZE and WRITE_SIZE, converted to bytes
 # with the factors a 1 GiB copy kernel gives for the same counters.
 PMC_STEPS_PER_LAUNCH = 224
-PMC_FETCH_BYTES_PER_LAUNCH = 31_344_952 * 2048  # counter reads 1 per 2 KiB fetched
+PMC_FETCH_BYTES_PER_LAUNCH = 31_344_830 * 2048  # counter reads 1 per 2 KiB fetched
 PMC_WRITE_BYTES_PER_LAUNCH = 541_326 * 1024     # counter reads 1 per KiB written
 
 
@@ -167,7 +167,7 @@ def main():
     steps_per_launch = sum(n for n, _, _ in r1["launches"]) / n_l
     achieved = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
     if persistent:
-        kernel = ("gh::persist_decode_kernel<3, 8, true, true>: one launch = one pick + step round per token "
+        kernel = ("gh::persist_decode_kernel<3, 8, true, true, false>: one launch = one pick + step round per token "
                   "for a whole run of steps")
     else:
         kernel = "every kernel of the decode round (one launch per fused op), timed as one span"
