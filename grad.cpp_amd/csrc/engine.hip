@@ -891,13 +891,15 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     std::memset(s.feed, 0, s.hist_stride * sizeof(unsigned long long));
     *s.stop_word = 0;
 
-    // Attention chunking: a (sequence, head) is split over several workgroups
-    // only while that is needed to cover the GPU (at least ~512 workgroups); a
-    // chunk is at most 1024 positions (the any-head-size kernel keeps its
-    // scores in LDS).
-    int chunk = 1024;
-    while (chunk > 128 && static_cast<long>(B) * sh.heads * ((sh.max_len + chunk - 1) / chunk) < 512)
-        chunk /= 2;
+    // Attention chunking: a (sequence, head) is split over several workgroups in
+    // runs of 512 cache positions, or 256 when that leaves fewer than ~192
+    // workgroups at a full context.  Longer runs win even when they leave compute
+    // units idle (measured at context 2048 with 2..16 sequences and at context 256
+    // with 8..64: every workgroup pays a dependent chain position -> page table ->
+    // cache rows -> merge, and a short run does not amortise it).
+    int chunk = 512;
+    if (static_cast<long>(B) * sh.heads * ((sh.max_len + chunk - 1) / chunk) < 192) chunk = 256;
+    if (o.flags & GH_FLAG_SMALL_ATTENTION_CHUNKS) chunk = 16;
     s.attn_chunk = chunk;
     s.attn_max_chunks = (sh.max_len + chunk - 1) / chunk;
     dev_alloc(s.attn_part, B * sh.heads * s.attn_max_chunks * (sh.head_size() + 2));

@@ -20,6 +20,7 @@ GH_OK, GH_ERR_RUNTIME, GH_ERR_OUT_OF_RANGE, GH_ERR_INVALID_ARGUMENT, GH_ERR_DEVI
 ENGINE_AUTO, ENGINE_GRAPH, ENGINE_EAGER, ENGINE_PERSISTENT = range(4)
 FLAG_PICK_GLOBAL_SCRATCH = 1
 FLAG_STEPWISE_PROMPT = 2
+FLAG_SMALL_ATTENTION_CHUNKS = 4
 
 
 class DeviceError(RuntimeError):

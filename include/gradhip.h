@@ -111,6 +111,12 @@ enum { GH_FLAG_PICK_GLOBAL_SCRATCH = 1 };
  * instead of pushing all prompt tokens through each layer at once. */
 enum { GH_FLAG_STEPWISE_PROMPT = 2 };
 
+/* Split every (sequence, head) of the decode attention into runs of 16 cache
+ * positions, each on a workgroup of its own, instead of the 256 or 512 the
+ * session would choose; for testing the merge of partial results at short
+ * contexts. */
+enum { GH_FLAG_SMALL_ATTENTION_CHUNKS = 4 };
+
 /* InferenceSession::InferenceSession (inference.cpp:121-148): allocates the
  * paged KV cache (2 * layers * max_len * d_model floats per sequence) and the
  * per-step scratch, and records the step graph. */

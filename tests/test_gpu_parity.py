@@ -79,6 +79,25 @@ def test_batched_step_equals_per_sequence_oracle(tiny_models, name, batch):
             assert_logits_close(got[b], oss[b].step(toks[b, t]), TOL, f"{name} B{batch} seq {b} step {t}")
 
 
+@pytest.mark.parametrize("batch", [1, 3])
+@pytest.mark.parametrize("name", ["hs64-gpt2", "hs64-modern", "odd-gpt2", "hs6-modern", "d256-modern"])
+def test_attention_split_over_workgroups_merges_to_the_same_logits(tiny_models, name, batch):
+    """Long contexts split a (sequence, head) over several workgroups whose partial softmax
+    states are merged by the last one to arrive; runs of 16 positions bring that to the tiny
+    shapes: up to three partial results per head, the last one ragged."""
+    cfg, W, om, gm = tiny_models[name]
+    gs = G.Session(gm, batch=batch, flags=G.FLAG_SMALL_ATTENTION_CHUNKS, page_tokens=8, shuffle_pages=True)
+    whole = G.Session(gm, batch=batch)
+    toks = synth.uniform_tokens(batch * cfg.max_len, cfg.vocab, 12).reshape(batch, cfg.max_len)
+    oss = [O.Session(om) for _ in range(batch)]
+    for t in range(cfg.max_len):
+        got, one = gs.step(toks[:, t]), whole.step(toks[:, t])
+        for b in range(batch):
+            ref = oss[b].step(toks[b, t])
+            assert_logits_close(got[b], ref, TOL, f"{name} B{batch} seq {b} step {t}")
+            assert_logits_close(got[b], one[b], 2e-5, f"{name} split vs whole, step {t}")
+
+
 @pytest.mark.parametrize("name", ["hs64-gpt2", "hs64-modern"])
 @pytest.mark.parametrize("batch", [1, 3])
 def test_prompt_pass_equals_steps(tiny_models, name, batch):
