@@ -108,7 +108,7 @@ class Config:
         return ((8 * self.d_model // 3) + 63) // 64 * 64
 
 
-# The shapes BASELINE.json's configs name (src/cli/presets.cpp:40-120 of grad.cpp).
+# The shapes of the benchmark configurations (src/cli/presets.cpp:40-120 of grad.cpp).
 PRESETS = {
     "c0": Config(ARCH_GPT2, 5000, 512, 6, 8, 96),
     "c1": Config(ARCH_GPT2, 16000, 768, 8, 12, 256),

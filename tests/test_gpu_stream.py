@@ -86,7 +86,7 @@ def test_stop_token_ends_the_run_and_the_next_call_continues(models, name):
     cfg, batch, gm, _ = models[name]
     ref = plain_run(gm, cfg, batch, N)
     # a token every sequence produces, chosen so that the run ends early: the id of
-    # sequence 0 at round 7, unless another sequence never picks it
+    # sequence 0's eighth pick, unless another sequence never picks it
     stop = int(ref[0, 7])
     last_first = max(int(np.flatnonzero(ref[b] == stop)[0]) if (ref[b] == stop).any() else N - 1
                      for b in range(batch))
