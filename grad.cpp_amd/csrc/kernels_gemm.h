@@ -163,14 +163,22 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) consume(a[u], b[u], gm[u]);
     }
-    for (; k < kq; k += 16) {
-        float4 a[MT], b[NT];
+    if (k < kq) {
+        // The steps left over go out as one more round with every load in flight: a
+        // step past the end re-reads the last one (a cache hit) and is not consumed.
+        float4 a[UNROLL][MT], b[UNROLL][NT], gm[UNROLL];
 #pragma unroll
-        for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const float4*>(wp[t] + k);
+        for (int u = 0; u < UNROLL - 1; u++) {
+            const int kk = min(k + 16 * u, kq - 16);
 #pragma unroll
-        for (int t = 0; t < MT; t++) a[t] = *reinterpret_cast<const float4*>(ap[t] + k);
-        const float4 g4 = RMS ? *reinterpret_cast<const float4*>(gp + k) : make_float4(1.f, 1.f, 1.f, 1.f);
-        consume(a, b, g4);
+            for (int t = 0; t < NT; t++) b[u][t] = *reinterpret_cast<const float4*>(wp[t] + kk);
+#pragma unroll
+            for (int t = 0; t < MT; t++) a[u][t] = *reinterpret_cast<const float4*>(ap[t] + kk);
+            gm[u] = RMS ? *reinterpret_cast<const float4*>(gp + kk) : make_float4(1.f, 1.f, 1.f, 1.f);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL - 1; u++)
+            if (k + 16 * u < kq) consume(a[u], b[u], gm[u]);
     }
     // Accumulator layout: lane holds column j, rows 4*g + r.
 #pragma unroll
