@@ -233,6 +233,205 @@ inline void launch_gemm16_as(const GemvParams& p, int M, hipStream_t st) {
                        st, p, M, m_groups);
 }
 
+// Weight tiles per workgroup of the wide kernel: 16000 rows = 250 workgroups.
+constexpr int kWideTiles = 4;
+
+// Wide projections of a few rows (the tied logits of a decode step: N = vocab,
+// M <= 32 sequences).  With 16 x 16 tiles every workgroup fetches its rows of A
+// again, and for N in the thousands that traffic (M x K per tile) is several
+// times the weights.  Here A is stationary: K is split over the 8 wavefronts of
+// a workgroup, each keeps its K / 8 slice of all M rows in registers in the MFMA
+// operand layout (RMSNorm gain already applied), and the workgroup walks
+// kWideTiles consecutive 16-row weight tiles, all requested at the start, so
+// every weight row crosses the chip once and A once per four tiles.
+// KS = K / 128 K-steps of 16 per wavefront; MT 16-row tiles of A.
+template <bool RMS, int MT, int KS>
+__global__ __launch_bounds__(512) void gemm_wide_kernel(const GemvParams p, int M) {
+    constexpr int KW = 8, NTILE = kWideTiles;
+    __shared__ float red[KW][MT][16 * 16];
+    __shared__ float ssq[KW][MT][16];
+    __shared__ float rinv[MT][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int K = p.K, kq = KS * 16;
+    const int j = lane & 15, g = lane >> 4;
+    const int fr = lane >> 2, fc = lane & 3;  // fetch layout: 4 lanes read 64 B of one row
+    const int from_lane = (j * 4 + g) * 4;
+    auto to_operand = [&](const float4& v) {
+        return make_float4(
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.x))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.y))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.z))),
+            __int_as_float(__builtin_amdgcn_ds_bpermute(from_lane, __float_as_int(v.w))));
+    };
+    const int n_tiles = (p.N + 15) >> 4;
+    const int tile0 = blockIdx.x * NTILE;
+    const int tile_end = min(tile0 + NTILE, n_tiles);
+    if (tile0 >= n_tiles) return;
+    // Weights and outputs go through bounded buffer descriptors: an access past the
+    // end reads zero / is dropped, so no load or store of the tile loop sits under
+    // a branch and the waits between them count exactly the operations in flight
+    // (a conditional one makes the compiler wait for everything, and a wavefront's
+    // loads return in order, so the tile being waited for would be the last).
+    constexpr unsigned kPastEnd = 0x80000000u;  // beyond any matrix this kernel is given
+    const __amdgpu_buffer_rsrc_t rs_w = make_buffer(p.W, static_cast<unsigned>(p.N) * K * 4u);
+    const __amdgpu_buffer_rsrc_t rs_o =
+        make_buffer(p.out, (static_cast<unsigned>(M - 1) * p.out_stride + p.N) * 4u);
+    auto fetch_tile = [&](int tile, float4 (&w)[KS]) {
+        const int row = tile * 16 + fr;
+        const unsigned off = (tile < tile_end && row < p.N)
+                                 ? (static_cast<unsigned>(row) * K + wave * kq + fc * 4) * 4u
+                                 : kPastEnd;
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_w, off, 64 * s, 0);
+            w[s] = make_float4(__int_as_float(v.x), __int_as_float(v.y), __int_as_float(v.z), __int_as_float(v.w));
+        }
+    };
+    // A first: a wavefront's loads return in the order they were issued, so the
+    // (cached) rows of A must not queue behind the weight tiles coming from HBM.
+    float4 as[MT][KS];  // this wavefront's K slice of every row
+    float4 gm[KS];
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        const float* ap = p.in + static_cast<size_t>(min(t * 16 + fr, M - 1)) * p.in_stride + wave * kq + fc * 4;
+#pragma unroll
+        for (int s = 0; s < KS; s++) as[t][s] = *reinterpret_cast<const float4*>(ap + 16 * s);
+    }
+#pragma unroll
+    for (int s = 0; s < KS; s++)
+        gm[s] = RMS ? *reinterpret_cast<const float4*>(p.gamma + wave * kq + 16 * s + g * 4)
+                    : make_float4(1.f, 1.f, 1.f, 1.f);
+    float4 wf[NTILE][KS];  // every tile of the workgroup is in flight from the start
+#pragma unroll
+    for (int f = 0; f < NTILE; f++) fetch_tile(tile0 + f, wf[f]);
+
+    // A moves to the operand layout once; RMSNorm's gain is applied here and the
+    // rows' sums of squares come from the same fragments.
+    {
+        float ss[MT];
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            ss[t] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const float4 a = to_operand(as[t][s]);
+                as[t][s] = a;
+                if (RMS) {
+                    ss[t] += dot4(a, a);
+                    as[t][s] = make_float4(a.x * gm[s].x, a.y * gm[s].y, a.z * gm[s].z, a.w * gm[s].w);
+                }
+            }
+        }
+        if (RMS) {
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float v = ss[t];
+                v += __shfl_xor(v, 16, kWave);
+                v += __shfl_xor(v, 32, kWave);
+                if (lane < 16) ssq[wave][t][lane] = v;
+            }
+            __syncthreads();
+            if (threadIdx.x < MT * 16) {
+                const int t = threadIdx.x >> 4, i = threadIdx.x & 15;
+                float ms = 0.0f;
+#pragma unroll
+                for (int w = 0; w < KW; w++) ms += ssq[w][t][i];
+                rinv[t][i] = 1.0f / sqrtf(ms / static_cast<float>(K) + kNormEps);
+            }
+            // the barrier inside the first tile orders rinv before its readers
+        }
+    }
+    // outputs of this thread in every tile: row m, column pair (jp, jp + 1)
+    const int e = threadIdx.x;
+    const int et = min(e >> 7, MT - 1), ei = (e & 127) >> 3, ejp = (e & 7) * 2;
+    const int em = et * 16 + ei;
+    const bool e_live = e < MT * 128 && em < M;
+
+    // Straight-line code over the tiles: no loop carries loads across a back edge,
+    // so every wait names exactly the tile it needs.  Tiles past the end were read
+    // as zeros and their stores are dropped.
+    {
+#pragma unroll
+        for (int f = 0; f < NTILE; f++) {
+            const int tile = tile0 + f;
+            v4f acc[MT];
+#pragma unroll
+            for (int t = 0; t < MT; t++) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const float4 b = to_operand(wf[f][s]);
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t][s].x, b.x, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t][s].y, b.y, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t][s].z, b.z, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t][s].w, b.w, acc[t], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) red[wave][t][(4 * g + r) * 16 + j] = acc[t][r];
+            __syncthreads();
+            const int n = tile * 16 + ejp;
+            {
+                const int at = ei * 16 + ejp;
+                float v0 = 0.0f, v1 = 0.0f;
+#pragma unroll
+                for (int w = 0; w < KW; w++) {
+                    v0 += red[w][et][at];
+                    v1 += red[w][et][at + 1];
+                }
+                if (RMS) {
+                    const float r = rinv[et][ei];
+                    v0 *= r;
+                    v1 *= r;
+                }
+                const unsigned o = (static_cast<unsigned>(em) * p.out_stride + n) * 4u;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(v0), rs_o, e_live && n < p.N ? o : kPastEnd, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(v1), rs_o,
+                                                      e_live && n + 1 < p.N ? o + 4u : kPastEnd, 0, 0);
+            }
+            __syncthreads();  // red is rewritten by the next tile
+        }
+    }
+    // the launch that makes the logits also ends the step (inference.cpp:256)
+    if (p.advance && blockIdx.x == 0 && threadIdx.x == 0) p.advance->pos += 1;
+}
+
+// The wide kernel takes a plain store without bias, K = 128 * KS (A fits in
+// registers) and matrices whose byte offsets stay below 2 GiB.
+inline bool gemm_wide_ok(const GemvParams& p, int M) {
+    // Up to 32 rows: at 64 the products (10 us of fp32 MFMA for 16000 x 768) bound
+    // the launch and the 16 x 16 tiling is as fast (measured 25.8 us either way).
+    if (p.N <= 8192 || M > 32 || p.K % 128 != 0 || p.bias != nullptr) return false;
+    if (static_cast<unsigned long long>(p.N) * p.K * 4ull >= 0x80000000ull) return false;
+    if ((static_cast<unsigned long long>(M - 1) * p.out_stride + p.N) * 4ull >= 0x80000000ull) return false;
+    const int ks = p.K / 128;
+    return ks == 4 || ks == 6 || ks == 8;
+}
+
+template <bool RMS, int MT, int KS>
+inline void launch_gemm_wide_as(const GemvParams& p, int M, hipStream_t st) {
+    const int n_tiles = (p.N + 15) / 16;
+    hipLaunchKernelGGL((gemm_wide_kernel<RMS, MT, KS>), dim3((n_tiles + kWideTiles - 1) / kWideTiles), dim3(512),
+                       0, st, p, M);
+}
+
+template <bool RMS, int MT>
+inline void launch_gemm_wide_ks(const GemvParams& p, int M, hipStream_t st) {
+    const int ks = p.K / 128;
+    if (ks == 8) launch_gemm_wide_as<RMS, MT, 8>(p, M, st);
+    else if (ks == 6) launch_gemm_wide_as<RMS, MT, 6>(p, M, st);
+    else launch_gemm_wide_as<RMS, MT, 4>(p, M, st);
+}
+
+template <bool RMS>
+inline void launch_gemm_wide(const GemvParams& p, int M, hipStream_t st) {
+    if (M <= 16) launch_gemm_wide_ks<RMS, 1>(p, M, st);
+    else launch_gemm_wide_ks<RMS, 2>(p, M, st);
+}
+
 // Tile shapes by measurement on the decode shapes (M = 64 rows): every launch
 // is bound by latency (kernel start, one trip to memory, the merge across the K
 // split), not by the weights, so small tiles on many workgroups win; long row
@@ -241,6 +440,9 @@ inline void launch_gemm16_as(const GemvParams& p, int M, hipStream_t st) {
 // each a multiple of 16.
 template <int EPI, bool RMS>
 inline void launch_gemm16(const GemvParams& p, int M, hipStream_t st) {
+    if constexpr (EPI == EPI_STORE) {
+        if (gemm_wide_ok(p, M)) return launch_gemm_wide<RMS>(p, M, st);
+    }
     const bool k8 = p.K % 128 == 0;
     if (p.N <= 1024 || M <= 16) {
         if (k8) launch_gemm16_as<EPI, RMS, 1, 1, 8>(p, M, st);
