@@ -239,10 +239,16 @@ __global__ __launch_bounds__(256) void attn_decode64_kernel(const AttnParams p) 
 
     float m = -INFINITY, lsum = 0.0f;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    // The page of a batch of 32 positions is looked up one batch ahead, beside the
+    // rows of the current batch: a lookup at the top of its own batch is one more
+    // trip to memory before that batch's rows can be requested.
+    int page = 0;
+    if (PAGE32 && t0 < t1) page = table[t0 >> shift];
     for (int tb = t0; tb < t1; tb += 32) {
         float4 k4[8], v4[8];
         size_t base = 0;
-        if (PAGE32) base = layer_base + static_cast<size_t>(table[tb >> shift]) * page_stride;
+        if (PAGE32) base = layer_base + static_cast<size_t>(page) * page_stride;
+        if (PAGE32 && tb + 32 < t1) page = table[(tb + 32) >> shift];
 #pragma unroll
         for (int it = 0; it < 8; it++) {
             const int tt = tb + it * 4 + sub;
