@@ -621,6 +621,36 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             }
             stamp();
 
+            // FFN1's operands (phase D).  Workgroups without a head spend phase C waiting
+            // for the attention of the others while HBM idles: their wavefronts that have no
+            // W_o row request the FFN1 rows now.  (The loads of a wavefront return in
+            // order, so its polls of phase C queue behind these rows; that wait is the
+            // long one anyway.  Workgroups with a head are late already and fetch as before.)
+            constexpr int NIT = MODERN ? F : F / 2;  // pairs of weight rows
+            float4 fw0[KD], fw1[KD];
+            NormRegs<KD> n2;
+            float fb0 = 0.0f, fb1 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < KD; i++) {
+                fw0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                fw1[i] = fw0[i];
+                n2.g[i] = fw0[i];
+                n2.b[i] = fw0[i];
+            }
+            auto load_ffn1 = [&]() {
+                if (first < NIT) {
+                    load_row<KD>(w.w1, 2 * first, D, lane, fw0);
+                    load_row<KD>(w.w1, 2 * first + 1, D, lane, fw1);
+                    load_norm<KD, PRO>(w.g2, w.be2, lane, n2);
+                    if (!MODERN) {
+                        fb0 = w.b1[2 * first];
+                        fb1 = w.b1[2 * first + 1];
+                    }
+                }
+            };
+            const bool early_ffn1 = wave >= (D + G - 1) / G && wg >= H;
+            if (early_ffn1) load_ffn1();
+
             // ===== phase C: x += b_o + attn @ W_o
             {
                 float4 w0[KD];
@@ -649,50 +679,30 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
 
             // ===== phase D: norm2 + FFN1 (SwiGLU or GELU) -> hidden cells
             {
-                constexpr int NIT = MODERN ? F : F / 2;  // pairs of weight rows
-                float4 w0[KD], w1[KD];
-                NormRegs<KD> n2;
-                float b0 = 0.0f, b1 = 0.0f;
-                if (first < NIT) {
-                    load_row<KD>(w.w1, 2 * first, D, lane, w0);
-                    load_row<KD>(w.w1, 2 * first + 1, D, lane, w1);
-                    load_norm<KD, PRO>(w.g2, w.be2, lane, n2);
-                    if (!MODERN) {
-                        b0 = w.b1[2 * first];
-                        b1 = w.b1[2 * first + 1];
-                    }
-                } else {
-#pragma unroll
-                    for (int i = 0; i < KD; i++) {
-                        w0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-                        w1[i] = w0[i];
-                        n2.g[i] = w0[i];
-                        n2.b[i] = w0[i];
-                    }
-                }
+                if (!early_ffn1) load_ffn1();
                 __syncthreads();  // every wave is done reading xs (phase C)
                 if (!gather_cells(p.xb, D, tag_of(l, 2), xs, p)) return;
                 for (int item = first; item < NIT; ) {
                     float4 h[KD];
                     load_input<KD, PRO>(xs, n2, lane, h);
-                    const float a = dot_row<KD>(w0, h);
-                    const float c = dot_row<KD>(w1, h);
+                    const float a = dot_row<KD>(fw0, h);
+                    const float c = dot_row<KD>(fw1, h);
                     if (lane == 0) {
                         const unsigned t = tag_of(l, 3);
                         if (MODERN) {
                             cell_put(p.hid + item, c * silu(a), t);
                         } else {
-                            cell_put(p.hid + 2 * item, gelu_tanh(a + b0), t);
-                            cell_put(p.hid + 2 * item + 1, gelu_tanh(c + b1), t);
+                            cell_put(p.hid + 2 * item, gelu_tanh(a + fb0), t);
+                            cell_put(p.hid + 2 * item + 1, gelu_tanh(c + fb1), t);
                         }
                     }
                     item += stride;
                     if (item < NIT) {
-                        load_row<KD>(w.w1, 2 * item, D, lane, w0);
-                        load_row<KD>(w.w1, 2 * item + 1, D, lane, w1);
+                        load_row<KD>(w.w1, 2 * item, D, lane, fw0);
+                        load_row<KD>(w.w1, 2 * item + 1, D, lane, fw1);
                         if (!MODERN) {
-                            b0 = w.b1[2 * item];
-                            b1 = w.b1[2 * item + 1];
+                            fb0 = w.b1[2 * item];
+                            fb1 = w.b1[2 * item + 1];
                         }
                     }
                 }
