@@ -370,6 +370,7 @@ struct Session {
 
     // persistent engine
     Cell* cells = nullptr;  // xa, xb, q, kn, vn, at (d each), hid (F), token (1)
+    size_t cells_count = 0;
     PersistCtl* ctl = nullptr;
     unsigned epoch = 1;         // tag base; grows with every step, never reused
     unsigned arrive_total = 0;  // logits phases completed so far
@@ -430,6 +431,36 @@ struct Session {
         if (stream) (void)hipStreamDestroy(stream);
     }
 };
+
+// The persistent kernel's workgroups wait for one another, so all of them have to
+// be resident at once: one per compute unit.  Two such launches in flight at the
+// same time (two sessions on two host threads) could each hold a part of the
+// GPU and wait for the rest for ever.  Every entry point that launches the
+// kernel therefore holds this process-wide lock from before the launch until
+// the stream has been synchronised; sessions on other engines never take it.
+static std::mutex g_persist_gate;
+
+static thread_local int g_gate_depth = 0;
+
+struct PersistGate {
+    std::unique_lock<std::mutex> lock;
+    explicit PersistGate(const struct Session& s);
+    ~PersistGate() {
+        if (lock.owns_lock()) g_gate_depth--;
+    }
+    PersistGate(const PersistGate&) = delete;
+    PersistGate& operator=(const PersistGate&) = delete;
+};
+
+PersistGate::PersistGate(const Session& s) {
+    if (s.engine != GH_ENGINE_PERSISTENT) return;
+    // a stream callback that calls into another persistent session would wait for itself
+    if (g_gate_depth > 0)
+        throw ApiError{GH_ERR_RUNTIME, "a persistent-engine call is already running on this thread "
+                                       "(token callbacks must not call into persistent-engine sessions)"};
+    lock = std::unique_lock<std::mutex>(g_persist_gate);
+    g_gate_depth++;
+}
 
 static KvLayout kv_layout(const Session& s) {
     return KvLayout{s.kv_pool,         s.page_table,           s.n_pages, s.pages_per_seq,
@@ -686,6 +717,18 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     const Model& m = *s.m;
     const Shape& sh = m.shape;
     if (n_steps <= 0 && n_picks <= 0) return;
+    // Tags are (epoch + step) * (layers + 1) * 8 + phase in 32 bits and are matched by
+    // equality, so they must not come round to a value a stale cell may still hold:
+    // long before that the cells are cleared on the stream (tag 0 is never used) and
+    // the epoch starts over.  Arrival counts are compared by wrap-safe difference.
+    {
+        const unsigned long long per_step = static_cast<unsigned long long>(sh.layers + 1) * 8ull;
+        const unsigned long long last = (static_cast<unsigned long long>(s.epoch) + n_steps + 2ull) * per_step + 8ull;
+        if (last >= 0xF0000000ull) {
+            HIP_CHECK(hipMemsetAsync(s.cells, 0, s.cells_count * sizeof(Cell), s.stream));
+            s.epoch = 1;
+        }
+    }
     PersistParams p{};
     p.E = m.E;
     p.P = m.P;
@@ -933,7 +976,14 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
             const size_t pick = (s.pick_row_in_lds ? V : 0) + kPickWorkFloats;
             s.persist_lds = std::max(work, pick) * sizeof(float);
             s.persist_grid = std::min(prop.multiProcessorCount, 256);
-            dev_alloc(s.cells, 6 * d + F + 1);
+            s.cells_count = 6 * d + F + 1;
+            dev_alloc(s.cells, s.cells_count);
+            // Rows of the cache written earlier in a launch by other workgroups are read
+            // with ordinary loads.  That is sound only because a row is never read before
+            // it is written and shares no 128-byte cache line with another row: rows are
+            // head_size floats from a base that hipMalloc aligns.
+            if ((sh.head_size() * sizeof(float)) % 128 != 0 || reinterpret_cast<uintptr_t>(s.kv_pool) % 256 != 0)
+                throw ApiError{GH_ERR_DEVICE, "persistent engine: cache rows are not whole 128-byte lines"};
             dev_alloc(s.ctl, 1);
             if (std::getenv("GRADHIP_PROF_DUMP")) {
                 s.prof_cap = 1 << 16;
@@ -1599,6 +1649,7 @@ gh_status gh_session_step(gh_session* sess, const int32_t* ids, float* logits_ho
     return guard([&] {
         if (!sess || !ids) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         Session& s = *sess->impl;
+        const PersistGate gate(s);  // held until this call has synchronised its launches
         check_capacity(s);
         check_ids(s, ids, s.B);
         const size_t V = s.m->shape.vocab;
@@ -1635,6 +1686,7 @@ gh_status gh_session_prefill(gh_session* sess, const int32_t* ids, int32_t len,
     return guard([&] {
         if (!sess || !ids) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         Session& s = *sess->impl;
+        const PersistGate gate(s);  // held until this call has synchronised its launches
         if (len < 0) throw ApiError{GH_ERR_INVALID_ARGUMENT, "negative length"};
         if (len == 0) return;
         if (s.pos + len > s.m->shape.max_len)
@@ -1664,6 +1716,7 @@ gh_status gh_session_score(gh_session* sess, const int32_t* ids, const int32_t* 
     return guard([&] {
         if (!sess || !ids || !targets || !nll_host) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         Session& s = *sess->impl;
+        const PersistGate gate(s);  // held until this call has synchronised its launches
         if (len < 0) throw ApiError{GH_ERR_INVALID_ARGUMENT, "negative length"};
         if (len == 0) return;
         if (s.pos + len > s.m->shape.max_len)
@@ -1787,6 +1840,7 @@ gh_status gh_session_decode(gh_session* sess, int32_t max_tokens, const gh_sampl
     return guard([&] {
         if (!sess || !opt || !out_count) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         Session& s = *sess->impl;
+        const PersistGate gate(s);  // held until this call has synchronised its launches
         check_sampling(*opt);
         *out_count = 0;
         s.timing = gh_timing{};
@@ -1825,6 +1879,7 @@ gh_status gh_session_decode_stream(gh_session* sess, int32_t max_tokens, const g
     return guard([&] {
         if (!sess || !opt || !out_count || !on_tokens) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         Session& s = *sess->impl;
+        const PersistGate gate(s);  // held until this call has synchronised its launches
         check_sampling(*opt);
         *out_count = 0;
         s.timing = gh_timing{};
@@ -1856,34 +1911,58 @@ gh_status gh_session_decode_stream(gh_session* sess, int32_t max_tokens, const g
             HIP_CHECK(hipEventRecord(s.ev[2], s.stream));
             bool kernel_done = false;
             unsigned idle = 0;
-            while (made < planned_picks) {
-                const unsigned long long w = __atomic_load_n(s.feed + made, __ATOMIC_ACQUIRE);
-                if (static_cast<unsigned>(w >> 32) == base + static_cast<unsigned>(made) + 1u) {
-                    const int32_t tok = static_cast<int32_t>(static_cast<unsigned>(w));
-                    if (tok < 0) break;  // the kernel saw the stop word before this pick
-                    if (out_ids) out_ids[made] = tok;
-                    const int32_t asked = on_tokens(user, &tok, made);
+            // Whatever ends this loop (the callback, a HIP error), the kernel must have
+            // stopped and the host's view must match the device's before control leaves.
+            auto settle = [&] {
+                stepped = std::min(made, planned_steps);
+                s.pos -= planned_steps - stepped;
+                s.arrive_total -= static_cast<unsigned>(planned_steps - stepped);
+                s.n_hist -= planned_picks - made;
+                s.picks -= planned_picks - made;
+            };
+            try {
+                while (made < planned_picks) {
+                    const unsigned long long w = __atomic_load_n(s.feed + made, __ATOMIC_ACQUIRE);
+                    if (static_cast<unsigned>(w >> 32) == base + static_cast<unsigned>(made) + 1u) {
+                        const int32_t tok = static_cast<int32_t>(static_cast<unsigned>(w));
+                        if (tok < 0) break;  // the kernel saw the stop word before this pick
+                        if (out_ids) out_ids[made] = tok;
+                        made++;  // delivered (or thrown out of) below: the round counts either way
+                        const int32_t asked = on_tokens(user, &tok, made - 1);
+                        idle = 0;
+                        if (asked != 0) __atomic_store_n(s.stop_word, 1u, __ATOMIC_RELEASE);
+                        if (tok == stop_token) break;  // the kernel ends after this token's step
+                        continue;
+                    }
+                    if (kernel_done) break;  // the launch is over and reported no further pick
+                    if ((++idle & 255u) == 0u) {
+                        const hipError_t q = hipStreamQuery(s.stream);
+                        if (q == hipSuccess) kernel_done = true;  // read the feed once more, then leave
+                        else if (q != hipErrorNotReady) HIP_CHECK(q);
+                    }
+                }
+            } catch (...) {
+                // stop the kernel at its next pick, wait for it, and take every round it
+                // still completed into account before handing the error on
+                __atomic_store_n(s.stop_word, 1u, __ATOMIC_RELEASE);
+                (void)hipStreamSynchronize(s.stream);
+                while (made < planned_picks) {
+                    const unsigned long long w = __atomic_load_n(s.feed + made, __ATOMIC_ACQUIRE);
+                    if (static_cast<unsigned>(w >> 32) != base + static_cast<unsigned>(made) + 1u
+                        || static_cast<int32_t>(static_cast<unsigned>(w)) < 0)
+                        break;
+                    if (out_ids) out_ids[made] = static_cast<int32_t>(static_cast<unsigned>(w));
                     made++;
-                    idle = 0;
-                    if (asked != 0) __atomic_store_n(s.stop_word, 1u, __ATOMIC_RELEASE);
-                    if (tok == stop_token) break;  // the kernel ends after this token's step
-                    continue;
                 }
-                if (kernel_done) break;  // the launch is over and reported no further pick
-                if ((++idle & 255u) == 0u) {
-                    const hipError_t q = hipStreamQuery(s.stream);
-                    if (q == hipSuccess) kernel_done = true;  // read the feed once more, then leave
-                    else if (q != hipErrorNotReady) HIP_CHECK(q);
-                }
+                settle();
+                if (du) s.picks = saved_picks + made;
+                *out_count = made;
+                throw;
             }
             HIP_CHECK(hipStreamSynchronize(s.stream));
             check_persist_abort(s);
             // persist_run advanced the host's view by the planned run: take back what was not run
-            stepped = std::min(made, planned_steps);
-            s.pos -= planned_steps - stepped;
-            s.arrive_total -= static_cast<unsigned>(planned_steps - stepped);
-            s.n_hist -= planned_picks - made;
-            s.picks -= planned_picks - made;
+            settle();
         } else {
             std::vector<char> seen(static_cast<size_t>(B), 0);
             int n_seen = 0;
@@ -1924,6 +2003,7 @@ gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t 
         if (!sess || !opt || !out_tokens || !out_len)
             throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         Session& s = *sess->impl;
+        const PersistGate gate(s);  // held until this call has synchronised its launches
         const Shape& sh = s.m->shape;
         check_sampling(*opt);
         *out_len = 0;

@@ -181,7 +181,8 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
                     v = __hip_atomic_load(&p.ctl->arrive[tid * 32], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                 for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-                if (__builtin_amdgcn_readfirstlane(v) >= target) break;
+                // wrap-safe: the counters run on for the life of the session
+                if (static_cast<int>(__builtin_amdgcn_readfirstlane(v) - target) >= 0) break;
                 ++spins;
                 if (spins > p.spin_limit
                     || ((spins & 63u) == 63u

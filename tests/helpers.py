@@ -29,17 +29,33 @@ def rel_err(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
-def assert_logits_close(got, ref, tol=1e-4, what=""):
-    """The logits rule: max|d| <= tol * max|ref| for the step, and per element
-    |d_i| <= tol * |ref_i| + 0.1 * tol * max|ref| (summation-order noise is
-    absolute, so an element near zero cannot be held to its own magnitude).
+# Worst observed values of the two logits rules per label, for the record a GPU
+# run prints at its end (tests/conftest.py).
+WORST = {}
+
+
+def assert_logits_close(got, ref, tol=1e-4, what="", abs_term=None):
+    """The per-step logits rule: max|d| <= tol * max|ref| for the step, and per
+    element |d_i| <= tol * max(|got_i|, |ref_i|) + abs_term (summation-order noise
+    is absolute, so an element near zero cannot be held to its own magnitude).
+    abs_term defaults to 5e-6 of the step's largest logit (the named configurations
+    stay below 1.5e-6 of it, the tiny shapes with livelier weights reach 3.2e-6).  (An absolute 1e-6 is
+    below the rounding of two correct fp32 implementations here: the 22M GPT-2
+    configuration has logits beyond 1.4, and its first step already differs from
+    the checker by 1.4e-6 on an element near zero while its max-norm error is 1e-6
+    relative.)
     grad.cpp's own parity test allows 1e-3 + 1e-3 * (|a| + |b|)
     (tests/integration/sanity_tests.cpp:322)."""
     e = rel_err(got, ref)
-    assert e <= tol, f"{what}: max|d|/max|ref| = {e:.3e} > {tol}"
     a, b = np.asarray(got, np.float64), np.asarray(ref, np.float64)
-    bad = np.abs(a - b) > tol * np.abs(b) + 0.1 * tol * np.abs(b).max()
-    assert not bad.any(), f"{what}: {int(bad.sum())} elements outside the per-element rule"
+    if abs_term is None:
+        abs_term = 5e-6 * float(np.abs(b).max())
+    per = float((np.abs(a - b) / (tol * np.maximum(np.abs(a), np.abs(b)) + abs_term)).max())
+    label = what.split(" step ")[0].split(" decode ")[0] or "unnamed"
+    w = WORST.setdefault(label, [0.0, 0.0])
+    w[0], w[1] = max(w[0], e / tol), max(w[1], per)
+    assert e <= tol, f"{what}: max|d|/max|ref| = {e:.3e} > {tol}"
+    assert per <= 1.0, f"{what}: per-element rule exceeded ({per:.3f} of the allowance)"
 
 
 def top2_margin(logits):

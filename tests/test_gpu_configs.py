@@ -15,6 +15,15 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-4  # per-step logits, relative to the step's largest logit
 
 
+def _teacher_forced(gm, om_logits, tokens, what):
+    """Steps a fresh session through `tokens` (the checker's stream) and holds the
+    logits of every step to the checker's: no step goes unchecked, whatever the
+    GPU's own loop would have picked at a near-tie."""
+    gs = G.Session(gm)
+    for i, t in enumerate(tokens):
+        assert_logits_close(gs.step([int(t)])[0], om_logits[i], TOL, f"{what} step {i}")
+
+
 @pytest.fixture(scope="module")
 def blas():
     return O.blas_init()
@@ -42,7 +51,8 @@ def test_c0_gpt2_small_greedy_80(blas):
         check_greedy_stream(got[0], ref, rsl, 16, f"c0 penalty {penalty}")
         if np.array_equal(got[0], ref):
             for i in range(96):
-                assert_logits_close(gsl[i, 0], rsl[i], TOL, f"c0 step {i}")
+                assert_logits_close(gsl[i, 0], rsl[i], TOL, f"c0 loop step {i}")
+        _teacher_forced(gm, rsl, ref[:96], f"c0 penalty {penalty}")
 
 
 def test_c1_gpt2_medium_per_step_logits(blas):
@@ -50,9 +60,7 @@ def test_c1_gpt2_medium_per_step_logits(blas):
     prompt = synth.uniform_tokens(32, cfg.vocab, 2001)
     ref, rsl = O.generate_greedy(om, prompt, 224, 1.0, want_logits=True)
     # teacher-forced on the oracle's tokens so every one of the 256 steps is compared
-    gs = G.Session(gm)
-    for i, t in enumerate(ref[:256]):
-        assert_logits_close(gs.step([t])[0], rsl[i], TOL, f"c1 step {i}")
+    _teacher_forced(gm, rsl, ref[:256], "c1")
     got = G.Session(gm).generate(prompt, 224, G.sampling(greedy=True, repetition_penalty=1.0))
     check_greedy_stream(got[0], ref, rsl, 32, "c1")
 
@@ -69,7 +77,8 @@ def test_c2_llama_sampled_224(llama):
     check_sampled_stream(got[0], ref, rsl, 32, u, opts, "c2")
     if np.array_equal(got[0], ref):
         for i in range(256):
-            assert_logits_close(gsl[i, 0], rsl[i], TOL, f"c2 step {i}")
+            assert_logits_close(gsl[i, 0], rsl[i], TOL, f"c2 loop step {i}")
+    _teacher_forced(gm, rsl, ref[:256], "c2")
     assert np.array_equal(gs.generate(prompt, 224, G.sampling(*opts), seed=3002), got)
 
 
@@ -85,6 +94,28 @@ def test_c3_llama_batch64_greedy(llama):
     for b in (0, 17, 63):
         ref, rsl = O.generate_greedy(om, prompts[b], 128, 1.0, want_logits=True)
         check_greedy_stream(got[b], ref, rsl, 128, f"c3 seq {b}")
+    # per-step logits at the full batch: two sequences followed by the checker, teacher-forced
+    # on the GPU's own picks (which must be the checker's arg-max unless that is a near-tie)
+    gs = G.Session(gm, batch=B)
+    last = gs.prefill(prompts)
+    watch = {b: O.Session(om) for b in (5, 40)}
+    refs = {}
+    for b, osess in watch.items():
+        for t in prompts[b]:
+            refs[b] = osess.step(int(t))
+        assert_logits_close(last[b], refs[b], TOL, f"c3 batch-64 prompt seq {b}")
+    for i in range(128):
+        nxt = gs.pick(opt)
+        for b in watch:
+            if nxt[b] != O.argmax_first(refs[b]):
+                srt = np.sort(refs[b])
+                assert srt[-1] - srt[-2] <= 4e-6 * np.abs(refs[b]).max(), f"c3 seq {b} token {i}"
+        if i == 127:
+            break
+        lg = gs.step(nxt)
+        for b, osess in watch.items():
+            refs[b] = osess.step(int(nxt[b]))
+            assert_logits_close(lg[b], refs[b], TOL, f"c3 batch-64 seq {b} step {i}")
     # every sequence equals its own batch-1 run on the GPU (batch invariance)
     single = G.Session(gm)
     for b in range(0, B, 7):

@@ -37,6 +37,40 @@ def test_interleaved_sessions_do_not_disturb_each_other(llama768):
         assert np.array_equal(lc[0], lc[2])
 
 
+def test_two_host_threads_each_decode_on_a_persistent_session(llama768):
+    """Sessions may live on different host threads.  Both run the one-launch engine,
+    whose workgroups wait for one another: the library has to keep two such launches
+    from sharing the GPU.  Each thread's stream must be the checker's."""
+    import threading
+    cfg, W, om, gm = llama768
+    prompts = [synth.uniform_tokens(9, cfg.vocab, 70 + i) for i in range(2)]
+    opt = G.sampling(greedy=True, repetition_penalty=1.0)
+    refs = [O.generate_greedy(om, p, 50, 1.0, want_logits=True) for p in prompts]
+    got, errs = [None, None], []
+
+    def work(i):
+        try:
+            s = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+            rounds = []
+            for _ in range(6):  # many launches per thread, so the two really interleave
+                rounds.append(s.generate(prompts[i], 50, opt)[0])
+            got[i] = rounds
+        except Exception as e:  # noqa: BLE001
+            errs.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errs, errs
+    from helpers import check_greedy_stream
+    for i in range(2):
+        for r in got[i]:
+            assert np.array_equal(r, got[i][0])
+        check_greedy_stream(got[i][0], refs[i][0], refs[i][1], 9, f"thread {i}")
+
+
 @pytest.mark.parametrize("batch", [7, 19, 33, 130])
 def test_batches_that_do_not_fill_a_tile(batch):
     cfg = synth.Config(synth.ARCH_MODERN, 301, 128, 2, 2, 24)
