@@ -1364,6 +1364,40 @@ static const float* stage_uniforms(Session& s, const float* uniforms, size_t n) 
     return s.uniforms;
 }
 
+// ---- a pick that allocates nothing (gh_pick_noalloc)
+
+// The sampler's working rows for callers that cannot allocate: one array per
+// GPU, held until the process ends.  Host code never uses this name as an
+// address; it asks the runtime where the array lives on the current device.
+constexpr size_t kNoAllocScratchFloats = size_t{1} << 20;  // 4 MiB
+static __device__ __align__(256) float scratch[kNoAllocScratchFloats];
+
+__global__ __launch_bounds__(kPickThreads) void pick_noalloc_kernel(const PickParams p, int* out_ids) {
+    extern __shared__ __attribute__((aligned(128))) float lds[];
+    const int b = blockIdx.x;
+    const int chosen = pick_body<false, kPickThreads>(p, b, p.work + static_cast<size_t>(b) * p.work_stride, lds);
+    if (threadIdx.x == 0) out_ids[b] = chosen;
+}
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current GPU, looked up once per device.
+static float* scratch_on_current_device() {
+    int dev = 0;
+    HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) throw ApiError{GH_ERR_DEVICE, "device index beyond the scratch table"};
+    std::lock_guard<std::mutex> lk(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+        if (!ptr) throw ApiError{GH_ERR_DEVICE, "the scratch array has no address on this device"};
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
 }  // namespace gh
 
 // ====================================================================== C ABI
@@ -2066,6 +2100,47 @@ gh_status gh_session_generate(gh_session* sess, const int32_t* prompts, int32_t 
     });
 }
 
+gh_status gh_pick_noalloc(const float* logits, int32_t batch, int32_t vocab, const int32_t* history,
+                          int32_t history_stride, int32_t n_history, const gh_sampling* opt,
+                          const float* uniforms, uint64_t seed, int32_t pick_index, int32_t* out_ids,
+                          void* hip_stream) {
+    return guard([&] {
+        if (!logits || !opt || !out_ids) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
+        if (batch < 1 || vocab < 1 || n_history < 0 || pick_index < 0 || n_history > history_stride
+            || (n_history > 0 && !history))
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "gh_pick_noalloc: bad sizes"};
+        check_sampling(*opt);
+        const size_t work_stride = (static_cast<size_t>(vocab) + kPickThreads + 3) / 4 * 4;
+        if (static_cast<size_t>(batch) * work_stride > kNoAllocScratchFloats)
+            throw ApiError{GH_ERR_INVALID_ARGUMENT,
+                           "gh_pick_noalloc: batch x (vocab + 1024) floats exceed the 4 MiB scratch array ("
+                               + std::to_string(kNoAllocScratchFloats) + " floats)"};
+        PickParams p{};
+        p.logits = logits;
+        p.work = scratch_on_current_device();
+        p.work_stride = static_cast<int>(work_stride);
+        p.V = vocab;
+        p.hist = const_cast<int*>(history);  // read only on this path
+        p.hist_stride = history_stride;
+        p.n_hist = n_history;
+        p.pick_idx = uniforms ? 0 : pick_index;
+        p.tok = nullptr;
+        p.temperature = opt->temperature;
+        p.top_k = opt->top_k;
+        p.top_p = opt->top_p;
+        p.penalty = opt->repetition_penalty;
+        p.greedy = opt->greedy;
+        p.uniforms = uniforms;
+        p.u_stride = 1;
+        p.seed_lo = static_cast<unsigned>(seed & 0xFFFFFFFFu);
+        p.seed_hi = static_cast<unsigned>(seed >> 32);
+        p.sort_cap = kPickWorkFloats;
+        hipLaunchKernelGGL(pick_noalloc_kernel, dim3(batch), dim3(kPickThreads), kPickWorkFloats * sizeof(float),
+                           static_cast<hipStream_t>(hip_stream), p, out_ids);
+        HIP_CHECK(hipGetLastError());
+    });
+}
+
 gh_status gh_session_last_timing(const gh_session* s, gh_timing* out) {
     return guard([&] {
         if (!s || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
@@ -2085,6 +2160,7 @@ gh_status gh_device_info(char* name, size_t name_len, int32_t* compute_units, in
         }
         if (compute_units) *compute_units = prop.multiProcessorCount;
         if (is_gfx950) *is_gfx950 = std::strstr(prop.gcnArchName, "gfx950") != nullptr;
+        (void)scratch_on_current_device();  // set-up for gh_pick_noalloc on this device
     });
 }
 

@@ -88,6 +88,8 @@ SYMBOLS = {
                                            TokenCallback, _vp, _i32p, _i32p]),
     "gh_session_generate": (C.c_int, [_vp, _i32p, C.c_int32, C.c_int32, C.POINTER(GhSampling), _f32p,
                                       C.c_uint64, _i32p, _i32p, _f32p, _i32p]),
+    "gh_pick_noalloc": (C.c_int, [_vp, C.c_int32, C.c_int32, _vp, C.c_int32, C.c_int32, C.POINTER(GhSampling), _vp,
+                                  C.c_uint64, C.c_int32, _vp, _vp]),
     "gh_session_last_timing": (C.c_int, [_vp, C.POINTER(GhTiming)]),
     "gh_tokenizer_load": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
     "gh_tokenizer_from_merges": (C.c_int, [_i32p, C.c_int32, C.POINTER(C.c_char_p), _i32p, C.c_int32,
@@ -147,6 +149,16 @@ def read_bandwidth(nbytes: int = 2 << 30, repeats: int = 5) -> float:
     out = C.c_double()
     _check(load_library().gh_device_read_bandwidth(nbytes, repeats, C.byref(out)))
     return out.value
+
+
+def pick_noalloc(logits_ptr: int, batch: int, vocab: int, history_ptr: int, history_stride: int, n_history: int,
+                 opt: GhSampling, out_ids_ptr: int, uniforms_ptr: int = 0, seed: int = 0, pick_index: int = 0,
+                 stream: int = 0) -> None:
+    """gh_pick_noalloc: every *_ptr is a DEVICE address (an int); enqueues the pick on
+    `stream` (a hipStream_t as an int, 0 = default stream) and returns without waiting."""
+    _check(load_library().gh_pick_noalloc(logits_ptr, batch, vocab, history_ptr or None, history_stride, n_history,
+                                          C.byref(opt), uniforms_ptr or None, seed, pick_index, out_ids_ptr,
+                                          stream or None))
 
 
 def _cfg_struct(cfg: synth.Config, fingerprint=None) -> GhConfig:

@@ -288,6 +288,26 @@ int32_t gh_codepoint_class(uint32_t codepoint);
 gh_status gh_session_score(gh_session* s, const int32_t* ids, const int32_t* targets, int32_t len,
                            float* nll_host);
 
+/* No counterpart in grad.cpp: gh_session_pick for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  Every pointer except opt is DEVICE memory owned by the caller:
+ * logits is batch x vocab, history is batch x history_stride token ids of which the
+ * first n_history of each row are read (the repetition penalty's window; may be NULL
+ * when n_history is 0), uniforms is one draw per sequence or NULL for the on-device
+ * Philox4x32-10(seed, sequence, pick_index), out_ids receives batch ids.  The kernel
+ * is enqueued on hip_stream (a hipStream_t, NULL for the default stream) and the call
+ * returns without waiting.  The sampler's working rows live in a 4 MiB array that is
+ * part of the library's code object (1,048,576 floats per GPU, held until the
+ * process ends): batch x (vocab + 1024, rounded up to 4) floats must fit, otherwise
+ * GH_ERR_INVALID_ARGUMENT.  The call makes no allocation of any kind after its first
+ * use on a device (which looks the array's address up; gh_device_info does the same
+ * look-up ahead of time).  All calls on one GPU share the array: calls that overlap
+ * in time on one GPU race; serialise them on one stream. */
+gh_status gh_pick_noalloc(const float* logits, int32_t batch, int32_t vocab, const int32_t* history,
+                          int32_t history_stride, int32_t n_history, const gh_sampling* opt,
+                          const float* uniforms, uint64_t seed, int32_t pick_index, int32_t* out_ids,
+                          void* hip_stream);
+
 /* ------------------------------------------------------------ measurement */
 
 /* GPU time of the last gh_session_generate call, from HIP events recorded on

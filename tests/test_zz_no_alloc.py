@@ -1,0 +1,82 @@
+"""gh_pick_noalloc, the entry point that allocates nothing: its picks must be those of
+gh_session_pick on the same logits, history, options and draws, on two calls in a row,
+the second with a smaller input (the shared working rows keep the first call's
+contents).  Device memory for the caller's side comes from torch."""
+import numpy as np
+import pytest
+
+import gradhip as G
+from gradhip import synth
+
+pytestmark = pytest.mark.gpu
+
+OPTIONS = [
+    dict(greedy=True, repetition_penalty=1.3),
+    dict(temperature=0.8, top_k=40, top_p=0.9, repetition_penalty=1.1),
+    dict(temperature=1.3, top_k=0, top_p=0.7, repetition_penalty=1.0),
+    dict(temperature=1.0, top_k=200, top_p=1.0, repetition_penalty=1.2),
+]
+
+
+def _case(torch, cfg, seed, batch, plen):
+    """Logits and history of `batch` sequences after a prompt, and the picks the
+    session entry point makes from them for every option set."""
+    W = synth.make_weights(cfg, seed, std=0.08)
+    gm = G.Model.from_tensors(cfg, W)
+    gs = G.Session(gm, batch=batch)
+    prompts = np.stack([synth.uniform_tokens(plen, cfg.vocab, seed + 1, stream=b) for b in range(batch)])
+    prompts[:, -3] = prompts[:, -1]  # a repeated token inside the penalty window
+    logits = gs.prefill(prompts)
+    u = synth.uniforms(batch, seed + 2)
+    want = [gs.pick(G.sampling(**o), uniforms=u).copy() for o in OPTIONS]
+    dev = dict(logits=torch.from_numpy(np.ascontiguousarray(logits)).cuda(),
+               hist=torch.from_numpy(np.ascontiguousarray(prompts.astype(np.int32))).cuda(),
+               u=torch.from_numpy(u.astype(np.float32)).cuda(),
+               out=torch.full((len(OPTIONS), batch), -7, dtype=torch.int32, device="cuda"))
+    return dev, want, batch, cfg.vocab, plen
+
+
+def _run(torch, dev, batch, vocab, plen):
+    for i, o in enumerate(OPTIONS):
+        G.pick_noalloc(dev["logits"].data_ptr(), batch, vocab, dev["hist"].data_ptr(), plen, plen,
+                       G.sampling(**o), dev["out"][i].data_ptr(), uniforms_ptr=dev["u"].data_ptr())
+    torch.cuda.synchronize()
+    return dev["out"].cpu().numpy()
+
+
+def test_noalloc_pick_equals_session_pick_twice_in_a_row():
+    torch = pytest.importorskip("torch")
+    G.device_info()  # the documented set-up call: looks the scratch array up on this device
+    big = _case(torch, synth.Config(synth.ARCH_MODERN, 50257, 128, 2, 2, 32), 900, 3, 12)
+    small = _case(torch, synth.Config(synth.ARCH_GPT2, 777, 128, 2, 2, 32), 910, 1, 9)
+    before = torch.cuda.memory_allocated()
+    got_big = _run(torch, *[big[0]], *big[2:])
+    got_small = _run(torch, *[small[0]], *small[2:])  # smaller rows over the first call's leftovers
+    got_big2 = _run(torch, *[big[0]], *big[2:])
+    assert torch.cuda.memory_allocated() == before
+    for i in range(len(OPTIONS)):
+        assert np.array_equal(got_big[i], big[1][i]), (OPTIONS[i], got_big[i], big[1][i])
+        assert np.array_equal(got_small[i], small[1][i]), (OPTIONS[i], got_small[i], small[1][i])
+        assert np.array_equal(got_big2[i], big[1][i])
+
+
+def test_noalloc_pick_philox_draws_and_limits():
+    torch = pytest.importorskip("torch")
+    cfg = synth.Config(synth.ARCH_MODERN, 1000, 128, 2, 2, 32)
+    W = synth.make_weights(cfg, 920, std=0.08)
+    gs = G.Session(G.Model.from_tensors(cfg, W))
+    prompt = synth.uniform_tokens(10, cfg.vocab, 921)
+    logits = gs.prefill(prompt[None, :])
+    opt = G.sampling(temperature=1.1, top_k=50, top_p=0.95, repetition_penalty=1.1)
+    want = gs.pick(opt, seed=77)  # the session's first pick: draw index 0 of stream (77, sequence 0)
+    lg = torch.from_numpy(np.ascontiguousarray(logits)).cuda()
+    hist = torch.from_numpy(prompt.astype(np.int32)).cuda()
+    out = torch.zeros(1, dtype=torch.int32, device="cuda")
+    G.pick_noalloc(lg.data_ptr(), 1, cfg.vocab, hist.data_ptr(), 10, 10, opt, out.data_ptr(), seed=77, pick_index=0)
+    torch.cuda.synchronize()
+    assert int(out.cpu()[0]) == int(want[0])
+    # beyond the array: refused with a clear message, nothing launched
+    with pytest.raises(ValueError, match="exceed the 4 MiB scratch"):
+        G.pick_noalloc(lg.data_ptr(), 64, 50257, hist.data_ptr(), 10, 10, opt, out.data_ptr())
+    with pytest.raises(ValueError):
+        G.pick_noalloc(lg.data_ptr(), 0, cfg.vocab, hist.data_ptr(), 10, 10, opt, out.data_ptr())
