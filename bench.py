@@ -3,8 +3,11 @@
 A step is one pass of the hot path over one batch: one new token for every
 sequence (pick on the GPU, then the whole transformer step).  The default
 workload is the 69M Llama block at batch 1 with the sampler the config names
-(temperature 0.8, top-k 40, top-p 0.9, repetition penalty 1.1); the 64-sequence
-batched decode of the same model is reported beside it.  Weights are seeded
+(temperature 0.8, top-k 40, top-p 0.9, repetition penalty 1.1), timed over
+--steps steps; the same workload as named (32 + 224), the two GPT-2 block
+workloads, the 64-sequence batched decode and the 2048-context decode are reported
+beside it, each with its fraction of the HBM roofline, and the CPU checker is timed
+on every one of them.  Weights are seeded
 N(0, 0.02), prompts seeded uniform ids; both live on the GPU before the clock
 starts.  Prints ONE JSON line.
 """
@@ -25,12 +28,16 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# rocprofv3 counters for one 224-step launch of the batch-1 persistent kernel
-# (32-token prompt already cached): FETCH_SIZE and WRITE_SIZE, converted to bytes
-# with the factors a 1 GiB copy kernel gives for the same counters.
-PMC_STEPS_PER_LAUNCH = 224
-PMC_FETCH_BYTES_PER_LAUNCH = 31_344_830 * 2048  # counter reads 1 per 2 KiB fetched
+# HBM traffic of the batch-1 persistent kernel, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE of a 224-step launch at contexts 33..256 (the counters converted to bytes
+# with the factors a 1 GiB copy kernel gives for them), as a ratio to the algorithmic
+# bytes of the same launch.  The kernel reads every weight once per step whatever the
+# number of steps, so the ratio carries over to other launch lengths; the summary named
+# here holds the commands and the raw counts.
+PMC_SOURCE = "profiles/persist_decode_kernel_c2_batch1.md"
+PMC_FETCH_BYTES_PER_LAUNCH = 31_345_339 * 2048  # counter reads 1 per 2 KiB fetched
 PMC_WRITE_BYTES_PER_LAUNCH = 541_326 * 1024     # counter reads 1 per KiB written
+PMC_ALGORITHMIC_BYTES_PER_LAUNCH = 63_406_751_744  # step_bytes() summed over that launch
 
 
 def step_bytes(cfg, batch, ctx):
@@ -81,26 +88,89 @@ def run_decode(G, synth, gm, cfg, batch, prompt_len, steps, warmup, opt, seed, e
             "prefill_tok_s": prefill_tok / (prefill_ms / 1e3) if prefill_ms else None}
 
 
-def cpu_baseline(synth, cfg, W, prompt, uniforms, opts):
-    """The CPU checker (a port of the reference's loop, BLAS-backed like it) timed
-    on this host: the full batch-1 workload once per thread setting."""
+def _cpu_run(O, om, prompt, n_new, pick, thread_plan):
+    """One sequence through the CPU checker, token by token like the reference's loop.
+    thread_plan: [(first_step, threads)], applied when that step is reached.  Returns
+    the seconds of every step() call."""
+    sess = O.Session(om)
+    plan = dict(thread_plan)
+    secs = np.zeros(len(prompt) + n_new)
+    toks = [int(t) for t in prompt]
+    logits = None
+    for i in range(len(prompt) + n_new):
+        if i in plan:
+            O.blas_set_threads(plan[i])
+        t0 = time.perf_counter()
+        if i >= len(prompt):
+            toks.append(pick(logits, toks, i - len(prompt)))
+        logits = sess.step(toks[i])
+        secs[i] = time.perf_counter() - t0
+    return secs
+
+
+def cpu_baseline(synth, W2):
+    """The CPU checker (a port of the reference's loop: one M=1 sgemm per projection,
+    BLAS-backed like it) timed on this host at 1 BLAS thread and at all of them (16 at
+    most), on every named workload.  The reference has no batch dimension, so c3 and c4
+    are one sequence each and their rate is the rate of any number of sequences run one
+    after another.  The pick is timed with the step it feeds."""
     import oracle_lib as O
     provider = O.blas_init()
-    om = O.Model.from_tensors(cfg, W)
-    T, k, p, pen = opts
-    out = {}
     ncpu = len(os.sched_getaffinity(0))
-    for threads in (1, min(ncpu, 16)):
-        O.blas_set_threads(threads)
-        t0 = time.perf_counter()
-        toks = O.generate_sample(om, prompt, uniforms, T, len(uniforms), pen, k, p)
-        dt = time.perf_counter() - t0
-        out[threads] = (len(toks)) / dt  # every step() call, prompt and decode alike
-    best = max(out, key=out.get)
-    return {"value": round(out[best], 2), "unit": "tok/s", "cores": best, "kind": "port",
-            "sample": f"32 prompt + {len(uniforms)} sampled decode steps of the batch-1 workload, "
-                      f"single pass per thread setting; BLAS: {provider.split(' [')[0].split('/')[-1]}",
-            "single_thread": round(out[1], 2), "host_cpus": ncpu}
+    nt = min(ncpu, 16)
+    opts = (0.8, 40, 0.9, 1.1)
+    u = synth.uniforms(224, 3002)
+
+    def greedy(penalty):
+        return lambda lg, toks, i: int(O.argmax_first(O.logits_with_penalty(lg, np.asarray(toks, np.int32), penalty)
+                                                      if penalty != 1.0 else lg))
+
+    def sampled(lg, toks, i):
+        adj = O.logits_with_penalty(lg, np.asarray(toks, np.int32), opts[3])
+        return int(O.sample_from_logits(adj, opts[0], opts[1], opts[2], float(u[i])))
+
+    out = {}
+    # (name, weights preset, prompt, new tokens, pick, seed)
+    plans = [("c0", "c0", 16, 80, greedy(1.2), 2000), ("c1", "c1", 32, 224, greedy(1.0), 2001),
+             ("c2", "c2", 32, 224, sampled, 2002), ("c3", "c2", 128, 128, greedy(1.0), 2003)]
+    for name, wname, n_prompt, n_new, pick, seed in plans:
+        cfg = synth.PRESETS[wname]
+        W = W2 if wname == "c2" else synth.make_weights(cfg, 1000 + int(wname[1]))
+        om = O.Model.from_tensors(cfg, W)
+        prompt = synth.uniform_tokens(n_prompt, cfg.vocab, seed)
+        rates = {}
+        for threads in (1, nt):
+            secs = _cpu_run(O, om, prompt, n_new, pick, [(0, threads)])
+            rates[threads] = {"prompt_tok_s": round(n_prompt / secs[:n_prompt].sum(), 2),
+                              "decode_tok_s": round(n_new / secs[n_prompt:].sum(), 2)}
+        out[name] = {"threads_1": rates[1], f"threads_{nt}": rates[nt],
+                     "sample": f"one sequence in full: {n_prompt} prompt steps + {n_new} decode steps"
+                               + ("; the reference runs the 64 sequences one after another at this rate"
+                                  if name == "c3" else "")}
+        del om
+    # c4: one sequence of 1536 + 512 steps costs about a minute on one thread, so the
+    # single-thread rate is taken on two windows of 32 steps (contexts 768.. and 2016..)
+    # of a pass that otherwise runs on all threads.
+    cfg4 = synth.PRESETS["c4"]
+    om = O.Model.from_tensors(cfg4, W2)
+    prompt = synth.uniform_tokens(1536, cfg4.vocab, 2004)
+    secs = _cpu_run(O, om, prompt, 512, greedy(1.0), [(0, nt), (768, 1), (800, nt), (2016, 1)])
+    many_prompt = np.r_[secs[:768], secs[800:1536]]
+    out["c4"] = {"threads_1": {"prompt_tok_s": round(32 / secs[768:800].sum(), 2),
+                               "decode_tok_s": round(32 / secs[2016:].sum(), 2)},
+                 f"threads_{nt}": {"prompt_tok_s": round(len(many_prompt) / many_prompt.sum(), 2),
+                                   "decode_tok_s": round(480 / secs[1536:2016].sum(), 2)},
+                 "sample": "one sequence of 1536 prompt + 512 decode steps on all threads, except steps "
+                           "768..799 (prompt) and 2016..2047 (decode), which run on one thread and give "
+                           "the single-thread rates at those contexts; 16 sequences run one after another "
+                           "at this rate"}
+    del om
+    O.blas_set_threads(nt)
+    best = max((1, nt), key=lambda t: out["c2"][f"threads_{t}"]["decode_tok_s"])
+    return {"value": out["c2"][f"threads_{best}"]["decode_tok_s"], "unit": "tok/s", "cores": best, "kind": "port",
+            "sample": "decode steps of the headline workload (c2: 32 prompt steps, then 224 sampled decode "
+                      f"steps), one pass per thread setting; BLAS: {provider.split(' [')[0].split('/')[-1]}",
+            "single_thread": out["c2"]["threads_1"]["decode_tok_s"], "host_cpus": ncpu, "configs": out}
 
 
 def main():
@@ -111,6 +181,7 @@ def main():
     ap.add_argument("--engine", default="auto", choices=["auto", "graph", "eager", "persistent"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-batch64", action="store_true", help="skip the batch-64 leg")
+    ap.add_argument("--no-small", action="store_true", help="skip the c0, c1 and c2-as-named legs")
     ap.add_argument("--only-batch64", action="store_true",
                     help="run only the batch-64 leg and print its object (for profiling that leg alone)")
     ap.add_argument("--no-long", action="store_true", help="skip the 2048-context leg")
@@ -169,6 +240,16 @@ def main():
                           "us_per_step_gpu": round(r4["gpu_ms"] * 1e3 / r4["steps"], 2),
                           "prefill_tok_s": round(r4["prefill_tok_s"], 1)}), flush=True)
         return
+    def roofline(r):
+        ach = r["bytes"] / (r["gpu_ms"] / 1e3) / 1e9
+        return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(ach / HBM_PEAK_GBS, 4)}
+
+    def leg(workload, r, batch):
+        return {"workload": workload, "value": round(batch * r["steps"] / r["wall_s"], 1), "unit": "tok/s",
+                "ms_per_step": round(r["wall_s"] * 1e3 / r["steps"], 5),
+                "prefill_tok_s": round(r["prefill_tok_s"], 1), "roofline": roofline(r)}
+
     r1 = run_decode(G, synth, gm, cfg, 1, 32, a.steps, a.warmup, sample, 2002, engine)
     tok_s = r1["steps"] / r1["wall_s"]
     persistent = r1["launches_per_step"] == 1
@@ -180,14 +261,16 @@ def main():
     if persistent:
         kernel = ("gh::persist_decode_kernel<3, 8, true, true, false>: one launch = one pick + step round per token "
                   "for a whole run of steps")
+        # measured HBM bytes per algorithmic byte of this kernel, times this launch's algorithmic bytes
+        traffic = int(bytes_per_launch * (PMC_FETCH_BYTES_PER_LAUNCH + PMC_WRITE_BYTES_PER_LAUNCH)
+                      / PMC_ALGORITHMIC_BYTES_PER_LAUNCH)
+        traffic_source = (f"{PMC_SOURCE}: FETCH_SIZE + WRITE_SIZE of a 224-step launch of this kernel are "
+                          f"{(PMC_FETCH_BYTES_PER_LAUNCH + PMC_WRITE_BYTES_PER_LAUNCH) / PMC_ALGORITHMIC_BYTES_PER_LAUNCH:.4f}"
+                          " of its algorithmic bytes; scaled to this launch's algorithmic bytes")
     else:
         kernel = "every kernel of the decode round (one launch per fused op), timed as one span"
-    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the
-    # summary under profiles/ for the command and the copy-kernel calibration);
-    # only valid for the launch shape it was measured on.
-    traffic = None
-    if persistent and steps_per_launch == PMC_STEPS_PER_LAUNCH:
-        traffic = PMC_FETCH_BYTES_PER_LAUNCH + PMC_WRITE_BYTES_PER_LAUNCH
+        traffic = int(bytes_per_launch)
+        traffic_source = "algorithmic bytes (no counter run covers this engine)"
 
     line = {
         "metric": "decode tok/s, 69M Llama block, batch 1",
@@ -200,6 +283,7 @@ def main():
         "device": info["name"],
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": traffic_source,
                      "kernel": kernel, "launches": n_l, "steps_per_launch": steps_per_launch,
                      "us_per_launch": round(us_per_launch, 1),
                      "bytes_per_launch": int(bytes_per_launch)},
@@ -211,39 +295,41 @@ def main():
     line["roofline"]["stream_read"] = round(stream, 1)
     line["roofline"]["frac_of_stream_read"] = round(achieved / stream, 4)
 
+    greedy = G.sampling(greedy=True, repetition_penalty=1.0)
+    if not a.no_small:
+        # the workload exactly as named, whatever --steps says: 32 prompt tokens, 224 sampled steps
+        rf = run_decode(G, synth, gm, cfg, 1, 32, 224, 224, sample, 2002, engine)
+        line["c2_full"] = leg("c2 as named: 32-token prompt, then 224 sampled decode steps (one launch)", rf, 1)
+        # c0 (the shape of the reference's own published figure) and c1
+        cfg0 = synth.PRESETS["c0"]
+        gm0 = G.Model.from_tensors(cfg0, synth.make_weights(cfg0, 1000))
+        r0 = run_decode(G, synth, gm0, cfg0, 1, 16, 80, 80, G.sampling(greedy=True, repetition_penalty=1.2),
+                        2000, engine)
+        line["c0"] = leg("c0: GPT-2 block 'small' (d512 L6 H8 F2048 V5000 C96), batch 1, 16-token prompt, "
+                         "80 greedy steps, repetition penalty 1.2 (the reference's default)", r0, 1)
+        del gm0
+        cfg1 = synth.PRESETS["c1"]
+        gm1 = G.Model.from_tensors(cfg1, synth.make_weights(cfg1, 1001))
+        r1m = run_decode(G, synth, gm1, cfg1, 1, 32, 224, 224, greedy, 2001, engine)
+        line["c1"] = leg("c1: GPT-2 block 'medium' (d768 L8 H12 F3072 V16000 C256), batch 1, 32-token prompt, "
+                         "224 greedy steps", r1m, 1)
+        del gm1
+
     if not a.no_batch64:
-        greedy = G.sampling(greedy=True, repetition_penalty=1.0)
         r64 = run_decode(G, synth, gm, cfg, 64, 128, 128, 16, greedy, 2003, engine)
-        ach64 = r64["bytes"] / (r64["gpu_ms"] / 1e3) / 1e9
-        line["batch64"] = {"workload": "c3: same model, 64 sequences, 128-token prompts, 128 greedy steps",
-                           "value": round(64 * r64["steps"] / r64["wall_s"], 1), "unit": "tok/s",
-                           "ms_per_step": round(r64["wall_s"] * 1e3 / r64["steps"], 4),
-                           "prefill_tok_s": round(r64["prefill_tok_s"], 1),
-                           "roofline": {"bound": "hbm", "achieved": round(ach64, 1), "peak": HBM_PEAK_GBS,
-                                        "unit": "GB/s", "frac": round(ach64 / HBM_PEAK_GBS, 4)}}
+        line["batch64"] = leg("c3: same model, 64 sequences, 128-token prompts, 128 greedy steps", r64, 64)
 
     if not a.no_long:
         # c4: same tensors, context 2048 (RoPE needs no table), 16 sequences with
         # 1536-token prompts in one pass, then greedy decode steps
         cfg4 = synth.PRESETS["c4"]
         gm4 = G.Model.from_tensors(cfg4, W)
-        greedy = G.sampling(greedy=True, repetition_penalty=1.0)
         r4 = run_decode(G, synth, gm4, cfg4, 16, 1536, 512, 16, greedy, 2004, engine)
-        ach4 = r4["bytes"] / (r4["gpu_ms"] / 1e3) / 1e9
-        line["context2048"] = {"workload": "c4: same weights, context 2048, 16 sequences, 1536-token prompts "
-                                           "in one pass, 512 greedy steps",
-                               "value": round(16 * r4["steps"] / r4["wall_s"], 1), "unit": "tok/s",
-                               "ms_per_step": round(r4["wall_s"] * 1e3 / r4["steps"], 4),
-                               "prefill_tok_s": round(r4["prefill_tok_s"], 1),
-                               "roofline": {"bound": "hbm", "achieved": round(ach4, 1), "peak": HBM_PEAK_GBS,
-                                            "unit": "GB/s", "frac": round(ach4 / HBM_PEAK_GBS, 4)}}
+        line["context2048"] = leg("c4: same weights, context 2048, 16 sequences, 1536-token prompts "
+                                  "in one pass, 512 greedy steps", r4, 16)
         del gm4
 
-    if not a.no_cpu:
-        prompt = synth.uniform_tokens(32, cfg.vocab, 2002)
-        line["cpu_baseline"] = cpu_baseline(synth, cfg, W, prompt, synth.uniforms(224, 3002), opts)
-    else:
-        line["cpu_baseline"] = None
+    line["cpu_baseline"] = None if a.no_cpu else cpu_baseline(synth, W)
     print(json.dumps(line), flush=True)
 
 
