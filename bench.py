@@ -193,7 +193,20 @@ def main():
     ap.add_argument("--stream-probe", action="store_true",
                     help="only time a plain read of 2 GiB (what a streaming kernel can reach of the "
                          "published HBM peak on this device) and exit")
+    ap.add_argument("--cache-probe", action="store_true",
+                    help="only time back-to-back re-reads of buffers from 32 MiB to 2 GiB (shows up to which "
+                         "size the memory-side cache serves a re-read) and exit")
     a = ap.parse_args()
+    if a.cache_probe:
+        import gradhip as G
+        rows = []
+        for mib in (1, 8, 32, 64, 96, 128, 160, 192, 224, 256, 288, 320, 384, 512, 768, 1024, 2048):
+            passes = max(8, min(200, (16 << 10) // mib))
+            rate = G.reread_bandwidth(mib << 20, passes)
+            rows.append({"MiB": mib, "passes": passes, "GBps": round(rate, 1),
+                         "us_per_pass": round((mib << 20) / rate / 1e3, 2)})
+        print(json.dumps({"reread": rows}))
+        return
     if a.stream_probe:
         import gradhip as G
         best = G.read_bandwidth(2 << 30, 5)

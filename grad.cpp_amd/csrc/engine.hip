@@ -1429,6 +1429,13 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const float4* __restri
             acc.w += v[u].w;
         }
     }
+    for (; i < n4; i += stride) {  // what is left (all of a buffer below 256 MiB)
+        const float4 v = a[i];
+        acc.x += v.x;
+        acc.y += v.y;
+        acc.z += v.z;
+        acc.w += v.w;
+    }
     if (acc.x + acc.y + acc.z + acc.w == 12345.0f) *sink = 1.0f;  // keeps the loads alive
 }
 
@@ -2183,7 +2190,7 @@ gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per
         } t;
         HIP_CHECK(hipMalloc(&t.buf, n4 * sizeof(float4)));
         HIP_CHECK(hipMalloc(&t.sink, sizeof(float)));
-        HIP_CHECK(hipMemset(t.buf, 0, n4 * sizeof(float4)));
+        HIP_CHECK(hipMemset(t.buf, 0x3c, n4 * sizeof(float4)));  // finite floats, not zeros
         HIP_CHECK(hipEventCreate(&t.e0));
         HIP_CHECK(hipEventCreate(&t.e1));
         double best = 0.0;
@@ -2198,6 +2205,45 @@ gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per
             if (r > 0) best = std::max(best, static_cast<double>(n4) * sizeof(float4) / (ms * 1e-3) / 1e9);
         }
         *gb_per_s = best;
+    });
+}
+
+gh_status gh_device_reread_bandwidth(size_t bytes, int32_t passes, double* gb_per_s) {
+    return guard([&] {
+        require_gpu();
+        if (!gb_per_s || bytes < (1u << 20) || passes < 1)
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "re-read bandwidth probe: need >= 1 MiB, >= 1 pass"};
+        const size_t n4 = bytes / sizeof(float4);
+        struct Scratch {
+            float4* buf = nullptr;
+            float* sink = nullptr;
+            hipEvent_t e0 = nullptr, e1 = nullptr;
+            ~Scratch() {
+                if (e0) (void)hipEventDestroy(e0);
+                if (e1) (void)hipEventDestroy(e1);
+                if (buf) (void)hipFree(buf);
+                if (sink) (void)hipFree(sink);
+            }
+        } t;
+        HIP_CHECK(hipMalloc(&t.buf, n4 * sizeof(float4)));
+        HIP_CHECK(hipMalloc(&t.sink, sizeof(float)));
+        HIP_CHECK(hipMemset(t.buf, 0x3c, n4 * sizeof(float4)));  // finite floats, not zeros
+        HIP_CHECK(hipEventCreate(&t.e0));
+        HIP_CHECK(hipEventCreate(&t.e1));
+        // Every pass is a launch of its own that streams the whole buffer (passes inside one
+        // launch would only re-read what the resident workgroups hold, which the L2s serve).
+        // 2048 x 256 threads with eight loads each cover 64 MiB per round.
+        const int grid = static_cast<int>(std::min<size_t>(8192, std::max<size_t>(256, n4 / (256 * 8))));
+        for (int r = -2; r < passes; r++) {  // two passes warm up, then one span over the rest
+            if (r == 0) HIP_CHECK(hipEventRecord(t.e0, nullptr));
+            hipLaunchKernelGGL(stream_read_kernel, dim3(grid), dim3(256), 0, nullptr, t.buf, n4, t.sink);
+        }
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipEventRecord(t.e1, nullptr));
+        HIP_CHECK(hipEventSynchronize(t.e1));
+        float ms = 0.0f;
+        HIP_CHECK(hipEventElapsedTime(&ms, t.e0, t.e1));
+        *gb_per_s = static_cast<double>(passes) * static_cast<double>(n4) * sizeof(float4) / (ms * 1e-3) / 1e9;
     });
 }
 

@@ -106,6 +106,7 @@ SYMBOLS = {
     "gh_codepoint_class": (C.c_int32, [C.c_uint32]),
     "gh_device_info": (C.c_int, [C.c_char_p, C.c_size_t, _i32p, _i32p]),
     "gh_device_read_bandwidth": (C.c_int, [C.c_size_t, C.c_int32, C.POINTER(C.c_double)]),
+    "gh_device_reread_bandwidth": (C.c_int, [C.c_size_t, C.c_int32, C.POINTER(C.c_double)]),
 }
 
 _lib = None
@@ -148,6 +149,13 @@ def read_bandwidth(nbytes: int = 2 << 30, repeats: int = 5) -> float:
     """GB/s of a plain streaming read of `nbytes` of device memory (best of `repeats`)."""
     out = C.c_double()
     _check(load_library().gh_device_read_bandwidth(nbytes, repeats, C.byref(out)))
+    return out.value
+
+
+def reread_bandwidth(nbytes: int, passes: int = 20) -> float:
+    """GB/s of `passes` back-to-back streaming reads of one buffer of `nbytes` (one timed span)."""
+    out = C.c_double(0.0)
+    _check(load_library().gh_device_reread_bandwidth(nbytes, passes, C.byref(out)))
     return out.value
 
 

@@ -330,6 +330,12 @@ gh_status gh_device_info(char* name, size_t name_len, int32_t* compute_units, in
  * can reach on this device, which is what roofline fractions are read against. */
 gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per_s);
 
+/* Measurement aid with no counterpart in grad.cpp: the same streaming kernel launched
+ * `passes` times back to back over one buffer of `bytes` (after two warm-up
+ * launches), timed as one span, launch gaps included.  A buffer that fits the memory-side cache is then
+ * served from it; the rate over a range of sizes shows where that stops. */
+gh_status gh_device_reread_bandwidth(size_t bytes, int32_t passes, double* gb_per_s);
+
 #ifdef __cplusplus
 }
 #endif
