@@ -173,6 +173,49 @@ def cpu_baseline(synth, W2):
             "single_thread": out["c2"]["threads_1"]["decode_tok_s"], "host_cpus": ncpu, "configs": out}
 
 
+def phase_stamps():
+    """Mean phase durations of one token of c2 on the persistent kernel, from the
+    stamps workgroup 0 leaves (GRADHIP_PROF_DUMP): per step one stamp after the pick,
+    five per layer, one when the logits rows have arrived, one at the end."""
+    import tempfile
+    dump = os.path.join(tempfile.mkdtemp(), "stamps.txt")
+    os.environ["GRADHIP_PROF_DUMP"] = dump
+    import gradhip as G
+    from gradhip import synth
+    cfg = synth.PRESETS["c2"]
+    gm = G.Model.from_tensors(cfg, synth.make_weights(cfg, 1002))
+    gs = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    gs.prefill(synth.uniform_tokens(32, cfg.vocab, 2002)[None, :])
+    gs.decode(224, G.sampling(0.8, 40, 0.9, 1.1), seed=2002)
+    gpu_us = gs.last_timing()["decode_ms"] * 1e3 / 224
+    gs.close()  # writes the dump
+    words = open(dump).read().split()
+    z = words.index("0")
+    st = np.array([int(x) for x in words[:z]], dtype=np.float64) / 100.0  # 100 MHz clock -> us
+    L = cfg.layers
+    period = 5 * L + 3
+    d = np.diff(st)
+    k = len(d) // period - 3
+    m = d[2 * period: (2 + k) * period].reshape(k, period).mean(axis=0)
+    lay = m[1:1 + 5 * L].reshape(L, 5).mean(axis=0)
+    pk = np.array([int(x) for x in words[z + 1:]], dtype=np.float64) / 100.0
+    pk = pk[: len(pk) // 3 * 3].reshape(-1, 3)[3:]
+    print(json.dumps({
+        "workload": "c2, one launch of 224 pick + step rounds, contexts 33..256", "steps_averaged": int(k),
+        "us_per_token_events": round(gpu_us, 2), "us_per_token_stamps": round(float(m.sum()), 2),
+        "pick_until_token_seen": round(float(m[0]), 2),
+        "pick_inside": {"wait_for_logits": round(float((pk[:, 1] - pk[:, 0]).mean()), 2),
+                        "penalty_sampler_token_out": round(float((pk[:, 2] - pk[:, 1]).mean()), 2)},
+        "layer_mean": {"embed_or_x_exchange+norm1+qkv": round(float(lay[0]), 2),
+                       "qkv_exchange+attention": round(float(lay[1]), 2),
+                       "attn_exchange+w_o": round(float(lay[2]), 2),
+                       "x_exchange+norm2+ffn1": round(float(lay[3]), 2),
+                       "hidden_exchange+ffn2": round(float(lay[4]), 2), "sum": round(float(lay.sum()), 2)},
+        "layers_total": round(float(lay.sum() * L), 2),
+        "x_exchange+logits_rows_arrive": round(float(m[-2]), 2),
+        "logits_dots_stores_arrival_count": round(float(m[-1]), 2)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -196,7 +239,14 @@ def main():
     ap.add_argument("--cache-probe", action="store_true",
                     help="only time back-to-back re-reads of buffers from 32 MiB to 2 GiB (shows up to which "
                          "size the memory-side cache serves a re-read) and exit")
+    ap.add_argument("--phase-stamps", action="store_true",
+                    help="only run one 224-step launch of the batch-1 workload with the persistent kernel's "
+                         "in-kernel phase stamps on (workgroup 0's clock at the end of every phase) and "
+                         "print the mean duration of every phase of a token")
     a = ap.parse_args()
+    if a.phase_stamps:
+        phase_stamps()
+        return
     if a.cache_probe:
         import gradhip as G
         rows = []
