@@ -985,6 +985,16 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
             if ((sh.head_size() * sizeof(float)) % 128 != 0 || reinterpret_cast<uintptr_t>(s.kv_pool) % 256 != 0)
                 throw ApiError{GH_ERR_DEVICE, "persistent engine: cache rows are not whole 128-byte lines"};
             dev_alloc(s.ctl, 1);
+            if (const char* near = std::getenv("GRADHIP_TEST_NEAR_WRAP")) {
+                // Test aid: start the session's two running counts `near` steps before the
+                // points where the arrival counters wrap around 2^32 and where the cell tags
+                // are re-based, so that a short run crosses both.
+                const unsigned n = static_cast<unsigned>(std::atoi(near));
+                s.arrive_total = (0u - n * static_cast<unsigned>(s.persist_grid)) / static_cast<unsigned>(s.persist_grid);
+                const unsigned sum = s.arrive_total * static_cast<unsigned>(s.persist_grid);
+                HIP_CHECK(hipMemcpy(&s.ctl->arrive[0], &sum, sizeof(sum), hipMemcpyHostToDevice));
+                s.epoch = static_cast<unsigned>(0xF0000000ull / (static_cast<unsigned long long>(sh.layers + 1) * 8ull)) - n;
+            }
             if (std::getenv("GRADHIP_PROF_DUMP")) {
                 s.prof_cap = 1 << 16;
                 dev_alloc(s.prof, s.prof_cap);

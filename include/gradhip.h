@@ -8,7 +8,10 @@
  * Threading: a model handle is immutable after creation and may be shared by
  * sessions on different host threads.  A session owns one HIP stream; calls on
  * one session must be serialised by the caller (grad.cpp's InferenceSession
- * and TextGen are not thread-safe either).
+ * and TextGen are not thread-safe either).  Sessions on the one-launch engine
+ * (batch 1, the shapes it is built for) take turns inside the library: its
+ * kernel needs the whole GPU, so a call that launches it holds a process-wide
+ * lock until the launch has finished; results do not depend on the order.
  *
  * There is no CPU fallback: every compute entry point fails with
  * GH_ERR_DEVICE when no gfx950 device is usable.

@@ -117,3 +117,26 @@ def test_unsupported_shapes_fall_back_or_refuse(models):
         G.Session(gm, engine=G.ENGINE_PERSISTENT)
     with pytest.raises(ValueError, match="persistent engine"):
         G.Session(models["llama-d768"][3], batch=2, engine=G.ENGINE_PERSISTENT)
+
+
+def test_counters_cross_their_wrap_points(models, monkeypatch):
+    """The arrival counters run on for the life of a session and wrap around 2^32; the
+    cell tags are re-based before they could repeat.  A session started a few steps
+    before both points decodes the same stream and logits as a fresh one."""
+    cfg, W, om, gm = models["llama-d768"]
+    prompt = synth.uniform_tokens(9, cfg.vocab, 77)
+    opt = G.sampling(0.9, 20, 0.95, 1.1)
+    ref, ref_logits = G.Session(gm, engine=G.ENGINE_PERSISTENT).generate(prompt, 60, opt, seed=4, want_logits=True)
+    monkeypatch.setenv("GRADHIP_TEST_NEAR_WRAP", "12")
+    near = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    monkeypatch.delenv("GRADHIP_TEST_NEAR_WRAP")
+    got, got_logits = near.generate(prompt, 60, opt, seed=4, want_logits=True)
+    assert np.array_equal(got, ref)
+    assert np.array_equal(got_logits, ref_logits)
+    # and step by step (one launch per step) across the same points
+    monkeypatch.setenv("GRADHIP_TEST_NEAR_WRAP", "5")
+    stepper = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    monkeypatch.delenv("GRADHIP_TEST_NEAR_WRAP")
+    fresh = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    for t in synth.uniform_tokens(20, cfg.vocab, 78):
+        assert np.array_equal(stepper.step([t]), fresh.step([t]))
