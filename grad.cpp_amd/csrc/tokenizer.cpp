@@ -1,7 +1,8 @@
 // Byte-level BPE tokenizer and GPT-2 pre-tokenizer (host code).  Follows the
 // behaviour of grad.cpp's src/tokenizer/pretokenize.cpp and byte_bpe.cpp; the
 // file format, fingerprint and message texts are the reference's, the
-// algorithms are written for this library.
+// algorithms are written for this library (the UTF-8 decoder is driven by a
+// lead-byte table, the splitter tries the pattern's alternatives in order).
 #include "tokenizer.h"
 
 #include "unicode_classes.h"
@@ -24,94 +25,114 @@ namespace pretok {
 
 CharClass classify(std::uint32_t cp) { return static_cast<CharClass>(unicode::class_of(cp)); }
 
+namespace {
+
+// What a lead byte promises: the sequence length (0: this byte cannot start a
+// sequence), the payload bits it carries itself, and the range its first
+// continuation byte must lie in.  The narrowed ranges are what makes the decoder
+// strict (RFC 3629): E0 and F0 refuse overlong forms, ED refuses surrogates, F4
+// refuses anything past U+10FFFF; C0, C1 and F5..FF promise nothing.
+struct LeadByte {
+    std::uint8_t length, payload_mask, second_lo, second_hi;
+};
+
+constexpr LeadByte lead_entry(unsigned b) {
+    if (b < 0x80) return {1, 0x7F, 0, 0};
+    if (b >= 0xC2 && b <= 0xDF) return {2, 0x1F, 0x80, 0xBF};
+    if (b >= 0xE0 && b <= 0xEF)
+        return {3, 0x0F, static_cast<std::uint8_t>(b == 0xE0 ? 0xA0 : 0x80), static_cast<std::uint8_t>(b == 0xED ? 0x9F : 0xBF)};
+    if (b >= 0xF0 && b <= 0xF4)
+        return {4, 0x07, static_cast<std::uint8_t>(b == 0xF0 ? 0x90 : 0x80), static_cast<std::uint8_t>(b == 0xF4 ? 0x8F : 0xBF)};
+    return {0, 0, 0, 0};
+}
+
+struct LeadTable {
+    LeadByte at[256];
+    constexpr LeadTable() : at{} {
+        for (unsigned b = 0; b < 256; b++) at[b] = lead_entry(b);
+    }
+};
+constexpr LeadTable kLead{};
+
+}  // namespace
+
+// Table-driven: the lead byte's entry says how many bytes to take and what the
+// second one may be; every further byte must be 10xxxxxx.  Anything else makes
+// the lead byte a scalar of its own (class Other), so the scan always advances.
 Scalar scalar_at(std::string_view text, std::size_t pos) {
-    const auto* s = reinterpret_cast<const unsigned char*>(text.data()) + pos;
-    const std::size_t left = text.size() - pos;
-    const unsigned char lead = s[0];
-    if (lead < 0x80) return {lead, 1, classify(lead)};
-    const Scalar bad{lead, 1, kOther};
-    // Sequence length and the allowed range of the second byte: the narrowed
-    // ranges exclude overlong forms (E0, F0), surrogates (ED) and anything past
-    // U+10FFFF (F4).
-    std::uint32_t len;
-    unsigned char lo = 0x80, hi = 0xBF;
-    std::uint32_t cp;
-    if (lead >= 0xC2 && lead <= 0xDF) {
-        len = 2;
-        cp = lead & 0x1Fu;
-    } else if ((lead & 0xF0) == 0xE0) {
-        len = 3;
-        cp = lead & 0x0Fu;
-        if (lead == 0xE0) lo = 0xA0;
-        if (lead == 0xED) hi = 0x9F;
-    } else if (lead >= 0xF0 && lead <= 0xF4) {
-        len = 4;
-        cp = lead & 0x07u;
-        if (lead == 0xF0) lo = 0x90;
-        if (lead == 0xF4) hi = 0x8F;
-    } else {
-        return bad;  // 80..C1 and F5..FF never start a sequence
+    const auto* bytes = reinterpret_cast<const unsigned char*>(text.data());
+    const LeadByte lead = kLead.at[bytes[pos]];
+    if (lead.length == 1) return {bytes[pos], 1, classify(bytes[pos])};
+    const Scalar lone{bytes[pos], 1, kOther};
+    if (lead.length == 0 || text.size() - pos < lead.length) return lone;
+    std::uint32_t cp = bytes[pos] & lead.payload_mask;
+    for (std::uint32_t k = 1; k < lead.length; k++) {
+        const unsigned char b = bytes[pos + k];
+        const unsigned char lo = k == 1 ? lead.second_lo : 0x80, hi = k == 1 ? lead.second_hi : 0xBF;
+        if (b < lo || b > hi) return lone;
+        cp = (cp << 6) | (b & 0x3Fu);
     }
-    if (left < len || s[1] < lo || s[1] > hi) return bad;
-    cp = (cp << 6) | (s[1] & 0x3Fu);
-    for (std::uint32_t k = 2; k < len; k++) {
-        if ((s[k] & 0xC0) != 0x80) return bad;
-        cp = (cp << 6) | (s[k] & 0x3Fu);
-    }
-    return {cp, len, classify(cp)};
+    return {cp, lead.length, classify(cp)};
 }
 
 namespace {
 
-// Length of a contraction ('s 't 'm 'd 're 've 'll, lower case only) at pos, or 0.
-std::size_t contraction_at(std::string_view text, std::size_t pos) {
-    if (text[pos] != '\'' || pos + 1 >= text.size()) return 0;
-    const char a = text[pos + 1];
-    if (a == 's' || a == 't' || a == 'm' || a == 'd') return 2;
-    if (pos + 2 >= text.size()) return 0;
-    const char b = text[pos + 2];
-    if ((a == 'r' && b == 'e') || (a == 'v' && b == 'e') || (a == 'l' && b == 'l')) return 3;
+// The split pattern, alternative by alternative, in the order a regex engine
+// tries them:  's|'t|'re|'ve|'m|'ll|'d | ?\p{L}+ | ?\p{N}+ | ?[^\s\p{L}\p{N}]+ | \s+(?!\S) | \s+
+// Each matcher returns the number of bytes it takes at pos, 0 when it does not match.
+
+// Bytes and scalars of the longest run of class `cls` starting at pos.
+struct Run {
+    std::size_t bytes = 0, scalars = 0, last_scalar_bytes = 0;
+};
+
+Run run_of(std::string_view text, std::size_t pos, CharClass cls) {
+    Run r;
+    while (pos + r.bytes < text.size()) {
+        const Scalar s = scalar_at(text, pos + r.bytes);
+        if (s.cls != cls) break;
+        r.bytes += s.length;
+        r.last_scalar_bytes = s.length;
+        r.scalars++;
+    }
+    return r;
+}
+
+// 's 't 're 've 'm 'll 'd: lower case only.
+std::size_t match_contraction(std::string_view text, std::size_t pos) {
+    static constexpr std::string_view kSuffixes[] = {"s", "t", "re", "ve", "m", "ll", "d"};
+    if (text[pos] != '\'') return 0;
+    const std::string_view rest = text.substr(pos + 1);
+    for (const std::string_view suffix : kSuffixes)
+        if (rest.substr(0, suffix.size()) == suffix) return 1 + suffix.size();
     return 0;
+}
+
+//  ?X+ for one of the three non-space classes: an optional U+0020, then the run.
+std::size_t match_spaced_run(std::string_view text, std::size_t pos, CharClass cls) {
+    const std::size_t lead_space = text[pos] == ' ' ? 1 : 0;
+    const Run run = run_of(text, pos + lead_space, cls);
+    if (run.scalars > 0) return lead_space + run.bytes;
+    return 0;  // without the space the run would have to start with a space of another class: no match either
+}
+
+// \s+(?!\S): white space not followed by text.  The greedy run gives back its last
+// scalar when text follows it, and fails when that leaves nothing.
+std::size_t match_space_before_space(std::string_view text, std::size_t pos) {
+    const Run run = run_of(text, pos, kSpace);
+    if (run.scalars == 0) return 0;
+    if (pos + run.bytes == text.size()) return run.bytes;
+    return run.bytes - run.last_scalar_bytes;  // 0 for a run of one scalar
 }
 
 }  // namespace
 
 std::size_t piece_end(std::string_view text, std::size_t pos) {
-    const std::size_t n = text.size();
-    if (const std::size_t c = contraction_at(text, pos)) return pos + c;
-
-    // A run of one class, which may take one leading space with it.
-    std::size_t at = pos;
-    Scalar head = scalar_at(text, at);
-    if (text[pos] == ' ' && pos + 1 < n) {
-        const Scalar after = scalar_at(text, pos + 1);
-        if (after.cls != kSpace) {
-            head = after;
-            at = pos + 1;
-        }
-    }
-    if (head.cls != kSpace) {
-        std::size_t end = at + head.length;
-        while (end < n) {
-            const Scalar s = scalar_at(text, end);
-            if (s.cls != head.cls) break;
-            end += s.length;
-        }
-        return end;
-    }
-
-    // White space.  `\s+(?!\S)` leaves the last white-space scalar of a run to
-    // the piece that follows when text follows the run; a run of one scalar,
-    // or one that ends the text, is a piece by itself (`\s+`).
-    std::size_t end = pos, last_start = pos, scalars = 0;
-    while (end < n) {
-        const Scalar s = scalar_at(text, end);
-        if (s.cls != kSpace) break;
-        last_start = end;
-        end += s.length;
-        scalars++;
-    }
-    return (end == n || scalars == 1) ? end : last_start;
+    if (const std::size_t n = match_contraction(text, pos)) return pos + n;
+    for (const CharClass cls : {kLetter, kNumber, kOther})
+        if (const std::size_t n = match_spaced_run(text, pos, cls)) return pos + n;
+    if (const std::size_t n = match_space_before_space(text, pos)) return pos + n;
+    return pos + run_of(text, pos, kSpace).bytes;  // \s+
 }
 
 }  // namespace pretok
