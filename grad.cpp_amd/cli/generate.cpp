@@ -2,16 +2,19 @@
 // checkpoint, on the GPU.  The command-line shape of `grad generate`
 // (src/cli/generate.cpp:61-107 of grad.cpp) for the part this library covers:
 //
-//   gradhip-generate <checkpoint> <tokenizer.tok> <prompt text>
+//   gradhip-generate <checkpoint> <tokenizer file> <prompt text>
+//   gradhip-generate <checkpoint> <prompt text> --corpus <corpus path> [--tokenizer v1|v2]
 //       [--max-tokens N] [--temperature T] [--top-k K] [--top-p P]
 //       [--repetition-penalty R] [--greedy] [--seed S]
 //
 // grad.cpp finds the tokenizer file from the corpus path and vocabulary size
-// (src/cli/common.cpp:160-187); here it is named explicitly.  The fingerprint
+// (src/cli/common.cpp:160-187); the second form does the same (resolve.h), the
+// first names the file.  The fingerprint
 // guard is the same: a checkpoint that records a tokenizer is only used with it.
 // Exit codes follow src/cli/main.cpp:94-103: 2 for a usage error, 1 for any failure.
 #include "gradhip.hpp"
 #include "options.h"
+#include "resolve.h"
 
 #include <iostream>
 #include <sstream>
@@ -37,18 +40,34 @@ std::string describe(const Options& o) {
 int main(int argc, char** argv) {
     try {
         const Options o = gradhip::cli::parse(argc, argv, Options{});
-        if (o.positional.size() != 3)
-            throw Usage("usage: gradhip-generate <checkpoint> <tokenizer.tok> <prompt> [options]");
-        const std::string &checkpoint = o.positional[0], &tokenizer_path = o.positional[1], &text = o.positional[2];
+        const bool by_corpus = o.corpus.has_value();
+        if (o.positional.size() != (by_corpus ? 2u : 3u))
+            throw Usage("usage: gradhip-generate <checkpoint> <tokenizer file> <prompt> [options]\n"
+                        "   or: gradhip-generate <checkpoint> <prompt> --corpus <corpus path> [--tokenizer v1|v2] [options]");
+        if (!by_corpus && o.tokenizer_flag) throw Usage("--tokenizer needs --corpus (the file is named otherwise)");
+        const std::string& checkpoint = o.positional[0];
+        const std::string& text = o.positional[by_corpus ? 1 : 2];
         std::cout << "\ngradhip Generation\n" << std::endl;
         const gradhip::GPTModel model = gradhip::GPTModel::load(checkpoint);
-        const std::unique_ptr<gradhip::Tokenizer> tokenizer = gradhip::load_tokenizer(tokenizer_path);
-        std::cout << "Tokenizer: " << tokenizer_path << " (" << gradhip::tokenizer_kind_flag(tokenizer->kind())
-                  << ", vocab " << tokenizer->vocab_size() << ")" << std::endl;
-        if (tokenizer->vocab_size() != model.getVocabSize()) {
-            throw std::runtime_error("tokenizer vocab " + std::to_string(tokenizer->vocab_size())
-                                     + " does not match the checkpoint's vocab of "
-                                     + std::to_string(model.getVocabSize()));
+        std::unique_ptr<gradhip::Tokenizer> tokenizer;
+        if (by_corpus) {
+            // load_for_inference (src/cli/common.cpp:346-358): the generation from the checkpoint,
+            // the flag and the files, then the file from the corpus path and the checkpoint's vocabulary
+            const gradhip::TokenizerKind kind = gradhip::cli::choose_tokenizer(
+                *o.corpus, model.getVocabSize(), gradhip::cli::parse_tokenizer_flag(o.tokenizer_flag), true,
+                model.getTokenizerFingerprint());
+            tokenizer = gradhip::cli::load_tokenizer_for_inference(*o.corpus, model.getVocabSize(), kind);
+            gradhip::cli::require_matching_vocab(*tokenizer, model.getVocabSize());
+        } else {
+            const std::string& tokenizer_path = o.positional[1];
+            tokenizer = gradhip::load_tokenizer(tokenizer_path);
+            std::cout << "Tokenizer: " << tokenizer_path << " (" << gradhip::tokenizer_kind_flag(tokenizer->kind())
+                      << ", vocab " << tokenizer->vocab_size() << ")" << std::endl;
+            if (tokenizer->vocab_size() != model.getVocabSize()) {
+                throw std::runtime_error("tokenizer vocab " + std::to_string(tokenizer->vocab_size())
+                                         + " does not match the checkpoint's vocab of "
+                                         + std::to_string(model.getVocabSize()));
+            }
         }
         gradhip::check_tokenizer_matches(model, *tokenizer, checkpoint);
         const std::vector<int> prompt = tokenizer->encode(text);

@@ -27,6 +27,11 @@ struct Options {
     std::optional<std::uint64_t> seed;
     bool stop_at_eos = false;   // not in grad.cpp: end a streamed reply at the tokenizer's end-of-text id
     bool keep_context = false;  // not in grad.cpp: chat lines continue one live context
+    // grad.cpp's way of naming the tokenizer: the corpus the checkpoint was trained on
+    // (a positional argument there) and --tokenizer v1|v2 (add_tokenizer_option,
+    // src/cli/common.cpp:148-150); the file follows from them and the checkpoint.
+    std::optional<std::string> corpus;
+    std::optional<std::string> tokenizer_flag;
 };
 
 template <class T>
@@ -66,6 +71,10 @@ inline Options parse(int argc, char** argv, Options o) {
             o.stop_at_eos = true;
         } else if (a == "--keep-context") {
             o.keep_context = true;
+        } else if (a == "--corpus") {
+            o.corpus = value();
+        } else if (a == "--tokenizer") {
+            o.tokenizer_flag = value();
         } else if (a == "--seed") {
             o.seed = number<std::uint64_t>(a, value());
         } else if (a.rfind("--", 0) == 0) {

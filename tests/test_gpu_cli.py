@@ -237,3 +237,32 @@ def test_generate_with_a_v1_tokenizer_cache(tmp_path):
     assert out.returncode == 1
     assert (f"Error: tokenizer v1:{other.fingerprint():016x} is not the one {tmp_path / 'm.bin'} was trained with "
             f"(v1:{v1.fingerprint():016x})").encode() in out.stderr
+
+
+def test_generate_finds_the_tokenizer_from_the_corpus_path(setup, tmp_path):
+    """`grad generate <checkpoint> <prompt> [corpus]` names no tokenizer file: it follows from the
+    corpus path, the checkpoint's vocabulary and its recorded tokenizer generation
+    (src/cli/common.cpp:346-358).  The same call shape here, with --corpus."""
+    d, tok, cfg, om = setup
+    corpus = tmp_path / "stories.txt"
+    corpus.write_text(TEXT)
+    tok_file = f"{corpus}.bytebpe_{tok.vocab_size}.tok"
+    open(tok_file, "wb").write(tok.file_image())
+    prompt = "the little cat"
+    out = run(d / "m.bin", prompt, "--corpus", corpus, "--max-tokens", 8, "--repetition-penalty", 1.1, "--greedy")
+    assert out.returncode == 0, out.stdout + out.stderr
+    greedy = O.generate_greedy(om, tok.encode(prompt.encode()), 8, 1.1)
+    assert f"Tokenizer: {tok_file} (v2, vocab {tok.vocab_size})\n".encode() in out.stdout
+    assert tok.decode(greedy) + b"\n" in out.stdout
+    # the flag may not contradict the checkpoint; a checkpoint without a record means v1, whose cache is not there
+    out = run(d / "m.bin", prompt, "--corpus", corpus, "--tokenizer", "v1", "--greedy")
+    assert out.returncode == 1
+    assert b"--tokenizer v1 does not match the checkpoint, which was trained with tokenizer v2:" in out.stderr
+    out = run(d / "plain.bin", prompt, "--corpus", corpus, "--greedy")
+    assert out.returncode == 1
+    assert (f"Error: No v1 tokenizer {corpus}.tokenizer_{tok.vocab_size}.cache; run: ./build/grad prepare {corpus} "
+            f"{tok.vocab_size} --tokenizer v1").encode() in out.stderr
+    out = run(d / "plain.bin", prompt, "--corpus", corpus, "--tokenizer", "v2", "--max-tokens", 3, "--greedy")
+    assert out.returncode == 0 and b"using the v2 tokenizer unverified" in out.stderr
+    assert run(d / "m.bin", prompt, "--corpus", corpus, "--tokenizer", "v3").returncode == 2
+    assert run(d / "m.bin", d / "t.tok", prompt, "--tokenizer", "v2").returncode == 2   # the flag needs --corpus
