@@ -2,17 +2,22 @@
 // non-overlapping windows, all positions of a batch of windows in one pass on the
 // GPU.  The scoring half of `grad eval` (src/cli/eval.cpp:44-133 of grad.cpp):
 //
-//   gradhip-eval <checkpoint> <tokens.bin> [--seq N] [--batches N]
+//   gradhip-eval <checkpoint> <tokens.bin> [--seq N] [--batches N] [--sampled [--seed S]] [--print-windows]
 //
 // <tokens.bin> is a "TOK1" file (include/grad/data/token_file.h:10-12: magic, u32
 // vocabulary size, u64 token count, u16 ids).  Window i covers tokens
 // [i * seq, i * seq + seq] (src/data/token_file.cpp:149-176), eight windows to a
 // batch (eval.cpp:77), loss = sum over batches of (batch mean x rows) / rows
 // (src/training/trainer.cpp:319-340).  --batches N scores the first N batches in file
-// order; grad.cpp draws a shuffled sample there (its std::shuffle order is
-// specific to the C++ library it was built with and is not reproduced).  The
-// split is named explicitly; grad.cpp derives both of its splits from a corpus
-// path and also reports bits per byte from the corpus size.
+// order; with --sampled the windows of every batch are drawn the way grad.cpp's
+// DataLoader draws them when `grad eval` is given --max-batches (eval.cpp:84-89,
+// src/data/dataloader.cpp:36-44): with replacement, std::uniform_int_distribution
+// over the window indices on a std::mt19937 seeded 20260921 for the validation
+// split (20260922 for the train split: --seed).  What that distribution returns
+// for given engine outputs is the C++ library's choice, so the sample equals
+// grad.cpp's when both are built with the same library; --print-windows lists
+// the indices drawn.  The split is named explicitly; grad.cpp derives both of
+// its splits from a corpus path and also reports bits per byte from the corpus size.
 #include "gradhip.hpp"
 
 #include <chrono>
@@ -21,6 +26,7 @@
 #include <fstream>
 #include <iomanip>
 #include <iostream>
+#include <random>
 #include <sstream>
 #include <string>
 #include <vector>
@@ -79,6 +85,8 @@ int main(int argc, char** argv) {
     try {
         std::vector<std::string> positional;
         int seq = 256, max_batches = 0;  // eval.cpp:140-141
+        bool sampled = false, print_windows = false;
+        unsigned seed = 20260921;  // eval.cpp:83
         for (int i = 1; i < argc; i++) {
             const std::string a = argv[i];
             const auto value = [&]() -> std::string {
@@ -87,10 +95,16 @@ int main(int argc, char** argv) {
             };
             if (a == "--seq") seq = to_int(a, value(), 1);
             else if (a == "--batches") max_batches = to_int(a, value(), 0);
+            else if (a == "--sampled") sampled = true;
+            else if (a == "--print-windows") print_windows = true;
+            else if (a == "--seed") seed = static_cast<unsigned>(to_int(a, value(), 0));
             else if (a.rfind("--", 0) == 0) throw Usage("unknown option " + a);
             else positional.push_back(a);
         }
-        if (positional.size() != 2) throw Usage("usage: gradhip-eval <checkpoint> <tokens.bin> [--seq N] [--batches N]");
+        if (positional.size() != 2)
+            throw Usage("usage: gradhip-eval <checkpoint> <tokens.bin> [--seq N] [--batches N] [--sampled [--seed S]] "
+                        "[--print-windows]");
+        if (sampled && max_batches == 0) throw Usage("--sampled needs --batches N (a sample of the whole split is the split)");
 
         std::cout << "\ngradhip Evaluation\n" << std::endl;
         const gradhip::GPTModel model = gradhip::GPTModel::load(positional[0]);
@@ -110,16 +124,29 @@ int main(int argc, char** argv) {
         double weighted = 0.0;
         size_t rows = 0;
         gh_session* full = nullptr;
+        std::mt19937 rng(seed);
         for (size_t b = 0; b < batches; b++) {
             const size_t first = b * kBatch;
             const int n = static_cast<int>(std::min<size_t>(kBatch, windows - first));
             std::vector<int32_t> ids(static_cast<size_t>(n) * seq), targets(ids.size());
+            std::vector<size_t> index(static_cast<size_t>(n));
+            for (int w = 0; w < n; w++) index[static_cast<size_t>(w)] = first + static_cast<size_t>(w);
+            if (sampled) {
+                std::uniform_int_distribution<size_t> pick(0, windows - 1);  // dataloader.cpp:40-44
+                for (int w = 0; w < n; w++) index[static_cast<size_t>(w)] = pick(rng);
+            }
+            if (print_windows) {
+                std::cout << "windows";
+                for (const size_t i : index) std::cout << " " << i;
+                std::cout << std::endl;
+            }
             for (int w = 0; w < n; w++) {
-                const std::uint16_t* win = file.tokens.data() + (first + w) * static_cast<size_t>(seq);
+                const size_t at = index[static_cast<size_t>(w)];
+                const std::uint16_t* win = file.tokens.data() + at * static_cast<size_t>(seq);
                 for (int t = 0; t <= seq; t++) {
                     if (win[t] >= file.vocab)  // token_file.cpp:164-170
                         throw std::runtime_error("token id " + std::to_string(win[t]) + " at offset "
-                                                 + std::to_string((first + w) * static_cast<size_t>(seq) + t)
+                                                 + std::to_string(at * static_cast<size_t>(seq) + t)
                                                  + " is outside the file's vocab of " + std::to_string(file.vocab));
                 }
                 for (int t = 0; t < seq; t++) {

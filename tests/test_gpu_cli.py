@@ -198,6 +198,23 @@ def test_eval_scores_a_token_file(setup, tmp_path):
                          capture_output=True, text=True, timeout=120)
     m = re.search(r"loss ([0-9.]+)  perplexity [0-9.]+  \((\d+) tokens", out.stdout)
     assert out.returncode == 0 and int(m.group(2)) == 8 * seq and abs(float(m.group(1)) - np.mean(batches[0])) <= 1e-3
+    # --sampled: windows drawn with replacement like grad.cpp's DataLoader under --max-batches; a few lines
+    # of C++ built with the same library give the draws to expect
+    draw = tmp_path / "draw.cpp"
+    draw.write_text("#include <cstdio>\n#include <random>\nint main() { std::mt19937 g(20260921); "
+                    "std::uniform_int_distribution<size_t> p(0, 10); "
+                    "for (int i = 0; i < 11; i++) std::printf(\"%zu \", p(g)); }\n")
+    subprocess.check_call(["g++", "-O1", str(draw), "-o", str(tmp_path / "draw")])
+    drawn = [int(x) for x in subprocess.check_output([str(tmp_path / "draw")], text=True).split()]
+    out = subprocess.run([exe, str(d / "m.bin"), str(path), "--seq", str(seq), "--batches", "2", "--sampled",
+                          "--print-windows"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    listed = [[int(x) for x in line.split()[1:]] for line in out.stdout.split("\n") if line.startswith("windows")]
+    assert listed == [drawn[:8], drawn[8:]] and len(set(drawn)) > 1
+    want = sum(np.mean([per_window[w] for w in b]) * len(b) for b in listed) / 11
+    m = re.search(r"loss ([0-9.]+)  perplexity [0-9.]+  \((\d+) tokens", out.stdout)
+    assert int(m.group(2)) == 11 * seq and abs(float(m.group(1)) - want) <= 1e-3
+    assert subprocess.run([exe, str(d / "m.bin"), str(path), "--sampled"], capture_output=True).returncode == 2
     # errors: a context longer than the model's, a file that is not a token file, the wrong vocabulary
     out = subprocess.run([exe, str(d / "m.bin"), str(path), "--seq", "65"], capture_output=True, text=True)
     assert out.returncode == 1 and "seq length exceeds the model's context (64)" in out.stderr
