@@ -123,8 +123,12 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
 #pragma unroll
         for (int u = 0; u < NT; u++) acc[t][u] = v4f{0.f, 0.f, 0.f, 0.f};
     }
-    // K-steps of loads in flight: as many as ~100 registers of fragments allow
-    constexpr int UNROLL = (MT + NT + 1) <= 3 ? 8 : (MT + NT + 1) <= 6 ? 4 : 2;
+    // K-steps of loads in flight per round.  Four, not as many as the registers would hold: with
+    // eight (16 x 16 tiles: 90-124 vector registers) fewer workgroups fit a compute unit, and a
+    // launch of these tiles lives on the number of loads the whole chip has in flight, not on
+    // one wavefront's (measured at 64 rows, 0.4385 -> 0.4345 ms per step, and at 16 rows,
+    // 0.568 -> 0.553 ms; two, three, five and six were all slower than four).
+    constexpr int UNROLL = (MT + NT + 1) <= 6 ? 4 : 2;
 
     auto consume = [&](const float4 (&a_in)[MT], const float4 (&b_in)[NT], const float4& g4) {
         float4 as[MT], b[NT];
@@ -432,6 +436,10 @@ inline void launch_gemm_wide(const GemvParams& p, int M, hipStream_t st) {
     else launch_gemm_wide_ks<RMS, 2>(p, M, st);
 }
 
+// At 64 rows (0.4575 ms per step with 2 x 1 tiles on 8 wavefronts for the wide projections and
+// 2 x 2 on 4 for the logits): wide 2 x 1 on 4 wavefronts 0.4384 (2 x 2 on 8: 0.4432, 1 x 4: 0.4504,
+// 2 x 4: 0.4742, 4 x 2: 0.4990, 2 x 1 on 2: 0.5125, 4 x 1 on 4: 0.5128); narrow 1 x 1 on 8 stays
+// (on 4: 0.4488, 2 x 1: 0.4615-0.5073); logits 2 x 4 on 8 0.4303 (2 x 2 on 8: 0.4351, 4 x 2: 0.4336).
 // Tile shapes by measurement on the decode shapes (M = 64 rows): every launch
 // is bound by latency (kernel start, one trip to memory, the merge across the K
 // split), not by the weights, so small tiles on many workgroups win; long row
@@ -448,10 +456,12 @@ inline void launch_gemm16(const GemvParams& p, int M, hipStream_t st) {
         if (k8) launch_gemm16_as<EPI, RMS, 1, 1, 8>(p, M, st);
         else launch_gemm16_as<EPI, RMS, 1, 1, 4>(p, M, st);
     } else if (p.N > 8192) {
-        if (M <= 64) launch_gemm16_as<EPI, RMS, 2, 2, 4>(p, M, st);
+        if (M <= 64 && k8) launch_gemm16_as<EPI, RMS, 2, 4, 8>(p, M, st);
+        else if (M <= 64) launch_gemm16_as<EPI, RMS, 2, 2, 4>(p, M, st);
         else launch_gemm16_as<EPI, RMS, 4, 2, 4>(p, M, st);
     } else if (M <= 64) {
-        if (k8) launch_gemm16_as<EPI, RMS, 2, 1, 8>(p, M, st);
+        // more than 32 rows: K over four wavefronts, twice as many (smaller) workgroups per compute unit
+        if (k8 && M <= 32) launch_gemm16_as<EPI, RMS, 2, 1, 8>(p, M, st);
         else launch_gemm16_as<EPI, RMS, 2, 1, 4>(p, M, st);
     } else {
         if (k8) launch_gemm16_as<EPI, RMS, 4, 1, 8>(p, M, st);
