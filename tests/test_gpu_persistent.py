@@ -15,6 +15,7 @@ SHAPES = {
     "gpt2-d512": synth.Config(synth.ARCH_GPT2, 1000, 512, 2, 8, 64),
     "gpt2-d768": synth.Config(synth.ARCH_GPT2, 700, 768, 2, 12, 72),
     "llama-d768": synth.Config(synth.ARCH_MODERN, 1200, 768, 2, 12, 96),
+    "gpt2-d1024": synth.Config(synth.ARCH_GPT2, 900, 1024, 2, 16, 48),
 }
 
 
