@@ -322,8 +322,11 @@ def main():
     steps_per_launch = sum(n for n, _, _ in r1["launches"]) / n_l
     achieved = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
     if persistent:
-        kernel = ("gh::persist_decode_kernel<3, 8, true, true, false>: one launch = one pick + step round per token "
-                  "for a whole run of steps")
+        # template arguments: d_model / 256, FFN width / 256, Llama block, sampler row in LDS (vocabularies
+        # up to ~38 k), not the streaming variant
+        kernel = (f"gh::persist_decode_kernel<{cfg.d_model // 256}, {cfg.d_ff // 256}, "
+                  f"{'true' if cfg.modern else 'false'}, {'true' if cfg.vocab <= 38000 else 'false'}, false>: "
+                  "one launch = one pick + step round per token for a whole run of steps")
         # measured HBM bytes per algorithmic byte of this kernel, times this launch's algorithmic bytes
         traffic = int(bytes_per_launch * (PMC_FETCH_BYTES_PER_LAUNCH + PMC_WRITE_BYTES_PER_LAUNCH)
                       / PMC_ALGORITHMIC_BYTES_PER_LAUNCH)
