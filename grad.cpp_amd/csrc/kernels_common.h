@@ -90,8 +90,10 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // Block-wide reductions through a small LDS scratch (one float per wave).
 // Every thread of the block must call them; all threads get the result.
-__device__ __forceinline__ float block_sum(float v, float* scratch) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+// nt: threads of the workgroup; a caller that knows it at compile time passes it
+// (blockDim.x is a load from the dispatch packet).
+__device__ __forceinline__ float block_sum(float v, float* scratch, int nt = blockDim.x) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (nt + 63) >> 6;
     v = wave_sum(v);
     __syncthreads();
     if (lane == 0) scratch[wave] = v;
@@ -101,8 +103,8 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     return r;
 }
 
-__device__ __forceinline__ float block_max(float v, float* scratch) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+__device__ __forceinline__ float block_max(float v, float* scratch, int nt = blockDim.x) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (nt + 63) >> 6;
     v = wave_max(v);
     __syncthreads();
     if (lane == 0) scratch[wave] = v;

@@ -96,6 +96,19 @@ __device__ __forceinline__ void coherent_store(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// "Did any thread of the workgroup give up its wait": a barrier and one LDS word
+// that stays zero until a wait is abandoned, after which the kernel only exits.
+// (__syncthreads_or reads the workgroup's dimensions from the dispatch packet on
+// every call: a trip to memory behind every exchange.)  The kernel clears the word
+// before its first wait.
+__shared__ unsigned g_wait_abandoned;
+
+__device__ __forceinline__ bool any_abandoned(bool failed) {
+    if (failed) g_wait_abandoned = 1u;
+    __syncthreads();
+    return g_wait_abandoned != 0u;
+}
+
 // Workgroup-wide: waits until cells [0, n) carry `tag`, copying the values to
 // dst (LDS).  Every thread polls only its own cells and stops as soon as they
 // have arrived; the workgroup meets once at the end.  Returns false when the wait
@@ -108,8 +121,10 @@ __device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float*
     bool failed = false;
     for (;;) {
         bool ok = true;
-        // two cells per 16-byte load, all of a thread's loads in flight together
-        for (int i = 2 * threadIdx.x; i < n; i += 2 * blockDim.x) {
+        // Two cells per 16-byte load.  The stride is the compile-time workgroup size:
+        // blockDim.x is a load from the dispatch packet, one more trip to memory in
+        // front of every poll.
+        for (int i = 2 * threadIdx.x; i < n; i += 2 * kPersistThreads) {
             const v4i w = coherent_load16(rs, static_cast<unsigned>(i) * 8u);
             ok = ok && w.y == itag && (i + 1 >= n || w.w == itag);
             dst[i] = __int_as_float(w.x);
@@ -124,7 +139,7 @@ __device__ inline bool gather_cells(const Cell* src, int n, unsigned tag, float*
             break;
         }
     }
-    if (__syncthreads_or(failed)) {
+    if (any_abandoned(failed)) {
         if (threadIdx.x == 0) {
             __hip_atomic_store(&p.ctl->where, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -148,9 +163,10 @@ __device__ __forceinline__ void feed_put(const PersistParams& p, int i_pick, int
 // learn the token from the cell.  False: the wait was abandoned.
 template <bool ROW_LDS, bool FEED>
 __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds, int i_pick,
-                                    unsigned arrive_gen, unsigned tok_tag, bool wait_logits) {
+                                    unsigned arrive_gen, unsigned tok_tag, bool wait_logits, int grid) {
     if (blockIdx.x != 0) return true;
-    const int tid = threadIdx.x;
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));  // nothing of the pick is computed ahead of the token loop
     if (p.prof && i_pick < 1024 && tid == 0) p.prof[p.prof_cap / 2 + 4 * i_pick + 2] = __builtin_amdgcn_s_memrealtime();
     PickParams pk = p.pick;
     pk.n_hist = p.pick.n_hist + i_pick;
@@ -173,7 +189,7 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
         // one wavefront watches the 16 arrival counters; the workgroup meets once
         bool failed = false;
         if (tid < 64) {
-            const unsigned target = arrive_gen * gridDim.x;
+            const unsigned target = arrive_gen * static_cast<unsigned>(grid);
             unsigned spins = 0;
             for (;;) {
                 unsigned v = 0;
@@ -192,7 +208,7 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
                 }
             }
         }
-        if (__syncthreads_or(failed)) {
+        if (any_abandoned(failed)) {
             if (tid == 0) {
                 __hip_atomic_store(&p.ctl->where, 0xFFFFFFFEu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -351,6 +367,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
 
     // The sequence's page table never changes while the kernel runs.
     for (int i = tid; i < p.kv.pages_per_seq; i += kPersistThreads) ptab[i] = p.kv.page_table[i];
+    if (tid == 0) g_wait_abandoned = 0u;
     __syncthreads();
     auto kv_at = [&](int layer, int which, int head, int t) -> size_t {
         const int page = ptab[t >> p.kv.page_shift];
@@ -369,7 +386,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         if ((!FEED || !ended) && i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick)) {
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
-            if (!persist_pick<ROW_LDS, FEED>(p, lds, i_pick, arrive_gen, tt, s > 0)) return;
+            if (!persist_pick<ROW_LDS, FEED>(p, lds, i_pick, arrive_gen, tt, s > 0, G)) return;
             i_pick++;
             if (wg == 0) {
                 // the pick used the whole LDS; restore the page table
@@ -516,7 +533,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                             }
                         }
                     }
-                    if (__syncthreads_or(failed)) {
+                    if (any_abandoned(failed)) {
                         if (tid == 0) {
                             __hip_atomic_store(&p.ctl->where, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                             __hip_atomic_store(&p.ctl->abort, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -72,10 +72,10 @@ __device__ __forceinline__ float key_float(unsigned k) {
 // One pass of the workgroup over v[0..n): f(i, v[i]) for i = tid, tid + nt, ...
 // Eight loads are issued before the first use, so a row in global memory costs
 // one memory latency per eight elements of a thread, not one per element.
-// f may store to v[i].
+// f may store to v[i].  nt: threads of the workgroup (a caller that knows it at
+// compile time passes it; blockDim.x is a load from the dispatch packet).
 template <class F>
-__device__ __forceinline__ void row_pass(const float* v, int n, F f) {
-    const int nt = blockDim.x;
+__device__ __forceinline__ void row_pass(const float* v, int n, F f, int nt = blockDim.x) {
     int i = threadIdx.x;
     for (; i + 7 * nt < n; i += 8 * nt) {
         float x[8];
@@ -138,16 +138,17 @@ __device__ __forceinline__ void select_bin_wave(const unsigned* hist, int want, 
     }
 }
 
-__device__ inline float kth_largest_lds(const float* v, int n, int k, unsigned* hist, unsigned* bcast) {
+__device__ inline float kth_largest_lds(const float* v, int n, int k, unsigned* hist, unsigned* bcast,
+                                        int nt = blockDim.x) {
     unsigned prefix = 0u, mask = 0u;
     int remaining = k;
     for (int shift = 24; shift >= 0; shift -= 8) {
-        for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0u;
+        for (int i = threadIdx.x; i < 256; i += nt) hist[i] = 0u;
         __syncthreads();
         // Keys cluster in a few bins (same sign and exponent), so lanes that hit
         // the same bin are counted with one atomic per wavefront.
-        const int n_round = (n + blockDim.x - 1) / blockDim.x * blockDim.x;
-        for (int i = threadIdx.x; i < n_round; i += blockDim.x) {
+        const int n_round = (n + nt - 1) / nt * nt;
+        for (int i = threadIdx.x; i < n_round; i += nt) {
             unsigned key = 0u;
             bool active = false;
             if (i < n) {
@@ -182,18 +183,19 @@ __device__ inline float kth_largest_lds(const float* v, int n, int k, unsigned* 
 // the k-th largest of the per-thread maxima is a lower bound T of the answer (at
 // least k elements are >= T), the elements >= T are few, and the answer is the
 // k-th largest of those.  Falls back to the radix select when k exceeds the
-// workgroup size or `work` (work_cap floats) cannot hold 2 * blockDim.x + 16.
+// workgroup size or `work` (work_cap floats) cannot hold 2 * nt + 16.
 __device__ __forceinline__ float kth_largest_block(const float* v, int n, int k, float* work, int work_cap,
-                                          unsigned* hist, unsigned* bcast, int* ishare) {
-    const int tid = threadIdx.x, nt = blockDim.x;
-    if (k > nt || work_cap < 2 * nt + 16) return kth_largest_lds(v, n, k, hist, bcast);
+                                          unsigned* hist, unsigned* bcast, int* ishare,
+                                          int nt = blockDim.x) {
+    const int tid = threadIdx.x;
+    if (k > nt || work_cap < 2 * nt + 16) return kth_largest_lds(v, n, k, hist, bcast, nt);
     float mx = -INFINITY;
-    row_pass(v, n, [&](int, float x) { mx = fmaxf(mx, x); });
+    row_pass(v, n, [&](int, float x) { mx = fmaxf(mx, x); }, nt);
     work[tid] = mx;
     if (tid == 0) ishare[1] = 0;
     __syncthreads();
     // one maximum per thread: a radix select over them is four short passes
-    const float T = kth_largest_lds(work, nt, k, hist, bcast);
+    const float T = kth_largest_lds(work, nt, k, hist, bcast, nt);
     __syncthreads();
     float* cand = work + nt;  // [nt + 16]
     row_pass(v, n, [&](int, float x) {
@@ -201,11 +203,11 @@ __device__ __forceinline__ float kth_largest_block(const float* v, int n, int k,
             const int slot = atomicAdd(&ishare[1], 1);
             if (slot < nt) cand[slot] = x;
         }
-    });
+    }, nt);
     __syncthreads();
     const int c = ishare[1];
     __syncthreads();
-    if (c > nt) return kth_largest_lds(v, n, k, hist, bcast);
+    if (c > nt) return kth_largest_lds(v, n, k, hist, bcast, nt);
     {
         const float mine = tid < c ? cand[tid] : -INFINITY;
         for (int j = c + tid; j < ((c + 15) & ~15); j += nt) cand[j] = -INFINITY;  // pad to 16
@@ -361,15 +363,20 @@ constexpr int kFastLdsFloats = 3 * kFastCandCap + 3 * 64 + 128;
 // (top-p) is formed in that order, lane by lane.
 // NT = threads of the workgroup and ROUNDS = elements per thread (compile time,
 // so that a thread's elements sit at immediate offsets and stay in registers
-// between the two passes); needs V <= ROUNDS * NT and V + NT readable floats
-// behind val.
+// between the two passes); needs V <= ROUNDS * NT.
 template <int NT, int ROUNDS>
 __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int k, float top_p, float u,
                                        float* work, float* red, int* ishare) {
     constexpr int nt = NT, nw = NT / 64;
     static_assert(ROUNDS <= 64, "one mask bit per element of a thread");
     static_assert(NT >= kFastCandCap, "every candidate needs a thread");
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Inside a kernel that picks once per iteration of a long loop, everything below
+    // that depends only on the thread and on V is loop-invariant; hoisted, the
+    // per-round masks alone are 2 * ROUNDS scalar registers, which end up spilled to
+    // scratch memory and reloaded one trip per round.  Opaque copies keep them here.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid), "+s"(V));
+    const int lane = tid & 63, wave = tid >> 6;
     if (V > ROUNDS * NT) return -1;
     float* cand_v = work;
     int* cand_i = reinterpret_cast<int*>(work + kFastCandCap);
@@ -380,16 +387,12 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
     int* perm = ridx + 64;                // [128]
 
     // element r * NT + tid of the row, scaled; -inf past the end
+    // (all reads first, at clamped offsets, so that they are in flight together)
     float x[ROUNDS];
-    const float* mine_base = val + tid;
 #pragma unroll
-    for (int r = 0; r < ROUNDS; r++) {
-        x[r] = -INFINITY;
-        if (r * NT < V) {  // uniform; the last round may read (and discard) floats just past V
-            const float raw = mine_base[r * NT];
-            x[r] = (tid < V - r * NT) ? raw * inv_t : -INFINITY;
-        }
-    }
+    for (int r = 0; r < ROUNDS; r++) x[r] = val[min(r * NT + tid, V - 1)];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; r++) x[r] = (tid < V - r * NT) ? x[r] * inv_t : -INFINITY;
     float mx = x[0];
 #pragma unroll
     for (int r = 1; r < ROUNDS; r++) mx = fmaxf(mx, x[r]);
@@ -526,8 +529,8 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
 // combined left to right, so the result is the serial sum up to regrouping.
 // parts: one float of LDS per wavefront.  Every thread must call these.
 template <class Get>
-__device__ inline float block_ordered_total(Get get, int n, float* parts) {
-    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+__device__ inline float block_ordered_total(Get get, int n, float* parts, int nt = blockDim.x) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
     // an odd run length: lane l starts at l * run, and an even stride would put
     // many lanes of a wavefront on the same LDS bank at every step of the walk
     const int run = ((n + nt - 1) / nt) | 1;
@@ -550,8 +553,9 @@ __device__ inline float block_ordered_total(Get get, int n, float* parts) {
 // First i in [0, n) whose running sum x(0) + ... + x(i) reaches thr, n when none
 // does.  slot: one int of LDS.
 template <class Get>
-__device__ inline int block_first_reach(Get get, int n, float thr, float* parts, int* slot) {
-    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6;
+__device__ inline int block_first_reach(Get get, int n, float thr, float* parts, int* slot,
+                                        int nt = blockDim.x) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // an odd run length: lane l starts at l * run, and an even stride would put
     // many lanes of a wavefront on the same LDS bank at every step of the walk
     const int run = ((n + nt - 1) / nt) | 1;
@@ -619,9 +623,9 @@ __device__ inline float top_p_cutoff(const float* val, int V, float top_p, float
             pmax = fmaxf(pmax, x[r]);
         }
     } else {
-        row_pass(val, V, [&](int, float v) { pmax = fmaxf(pmax, v); });
+        row_pass(val, V, [&](int, float v) { pmax = fmaxf(pmax, v); }, nt);
     }
-    pmax = block_max(pmax, red);
+    pmax = block_max(pmax, red, nt);
     __shared__ float sums[2][kPickThreads / 64];
     int calls = 0;
     auto upper_mass = [&](unsigned key) {
@@ -631,7 +635,7 @@ __device__ inline float top_p_cutoff(const float* val, int V, float top_p, float
 #pragma unroll
             for (int r = 0; r < ROUNDS; r++) mass += (x[r] >= t) ? x[r] : 0.0f;
         } else {
-            row_pass(val, V, [&](int, float v) { mass += (v >= t) ? v : 0.0f; });
+            row_pass(val, V, [&](int, float v) { mass += (v >= t) ? v : 0.0f; }, nt);
         }
         // block sum with one barrier per call: successive calls alternate between two
         // sets of per-wavefront slots
@@ -692,8 +696,11 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
     __shared__ int ishare[2];
 
     constexpr int nt = NT;
-    const int tid = threadIdx.x;
-    const int V = p.V;
+    // Opaque copies, as in sample_topk_fast: nothing derived from them is computed
+    // ahead of a caller's loop and kept in registers through it.
+    int tid = threadIdx.x;
+    int V = p.V;
+    asm volatile("" : "+v"(tid), "+s"(V));
     const float* logits = p.logits + static_cast<size_t>(b) * V;
     const int* hist = p.hist + static_cast<size_t>(b) * p.hist_stride;
 
@@ -727,7 +734,7 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
             }
         }
     } else {
-        row_pass(logits, V, [&](int i, float v) { val[i] = v; });
+        row_pass(logits, V, [&](int i, float v) { val[i] = v; }, nt);
     }
     if (tid < window) win_tok[tid] = window_token;
     if (tid < 64) {
@@ -772,7 +779,7 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
                 best = v;
                 bi = i;
             }
-        });
+        }, nt);
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
             const float ov = __shfl_xor(best, o, kWave);
@@ -811,10 +818,10 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
             __syncthreads();
             if (c >= 0) return c;
         }
-        row_pass(val, V, [&](int i, float v) { val[i] = v * inv_t; });
+        row_pass(val, V, [&](int i, float v) { val[i] = v * inv_t; }, nt);
         __syncthreads();
         if (p.top_k > 0 && p.top_k < V) {
-            const float thr = kth_largest_block(val, V, p.top_k, srt, p.sort_cap, hist256, bcast, ishare);
+            const float thr = kth_largest_block(val, V, p.top_k, srt, p.sort_cap, hist256, bcast, ishare, nt);
             // Survivors of the cut (ties at the threshold included).  When they fit
             // one wavefront the rest of the sampler runs there.
             int* cidx = reinterpret_cast<int*>(srt);
@@ -825,7 +832,7 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
                     const int slot = atomicAdd(&ishare[1], 1);
                     if (slot < 64) cidx[slot] = i;
                 }
-            });
+            }, nt);
             __syncthreads();
             const int S0 = ishare[1];
             if (S0 <= 64 && p.sort_cap >= 512) {
@@ -840,21 +847,21 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
             }
             row_pass(val, V, [&](int i, float v) {
                 if (v < thr) val[i] = -1e10f;
-            });
+            }, nt);
             __syncthreads();
         }
         float m = -INFINITY;
-        row_pass(val, V, [&](int, float v) { m = fmaxf(m, v); });
-        m = block_max(m, red);
+        row_pass(val, V, [&](int, float v) { m = fmaxf(m, v); }, nt);
+        m = block_max(m, red, nt);
         float sum = 0.0f;
         row_pass(val, V, [&](int i, float v) {
             const float e = expf(v - m);
             val[i] = e;
             sum += e;
-        });
-        sum = block_sum(sum, red);
+        }, nt);
+        sum = block_sum(sum, red, nt);
         const float inv_sum = 1.0f / sum;
-        row_pass(val, V, [&](int i, float v) { val[i] = v * inv_sum; });
+        row_pass(val, V, [&](int i, float v) { val[i] = v * inv_sum; }, nt);
 
         if (p.top_p < 1.0f) {
             float cutoff;
@@ -863,7 +870,7 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
             else cutoff = top_p_cutoff<0, 1>(val, V, p.top_p, red);
             row_pass(val, V, [&](int i, float v) {
                 if (v < cutoff) val[i] = 0.0f;
-            });
+            }, nt);
         }
         __syncthreads();
 
@@ -874,14 +881,14 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
         float total = 1.0f;
         bool divide = false;
         if (renorm) {
-            total = block_ordered_total([&](int q) { return val[q]; }, V, parts);
+            total = block_ordered_total([&](int q) { return val[q]; }, V, parts, nt);
             divide = total > 0.0f;
         }
         if (u <= 0.0f) {
             if (tid == 0) ishare[0] = 0;
         } else {
-            const int at = divide ? block_first_reach([&](int q) { return val[q] / total; }, V, u, parts, &ishare[1])
-                                  : block_first_reach([&](int q) { return val[q]; }, V, u, parts, &ishare[1]);
+            const int at = divide ? block_first_reach([&](int q) { return val[q] / total; }, V, u, parts, &ishare[1], nt)
+                                  : block_first_reach([&](int q) { return val[q]; }, V, u, parts, &ishare[1], nt);
             if (tid == 0) ishare[0] = at < V ? at : V - 1;
         }
         __syncthreads();
