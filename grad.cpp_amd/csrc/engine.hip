@@ -141,11 +141,9 @@ struct Model {
     float *gf = nullptr, *bf = nullptr;
     float *rope_cos = nullptr, *rope_sin = nullptr;  // (max_len, head_size/2)
     std::vector<Placement> place;                    // file order
-    LayerPtrs* d_layers = nullptr;                   // the layer table, on the device
 
     ~Model() {
         if (blob) (void)hipFree(blob);
-        if (d_layers) (void)hipFree(d_layers);
     }
 };
 
@@ -265,14 +263,6 @@ static std::unique_ptr<Model> upload_model(const Shape& shape, const std::vector
     }
     HIP_CHECK(hipFree(stage));
 
-    {
-        std::vector<LayerPtrs> table;
-        for (const LayerWeights& w : m->layers)
-            table.push_back({w.wqkv, w.bqkv, w.wo, w.bo, w.w1, w.b1, w.w2, w.b2, w.g1, w.be1, w.g2, w.be2});
-        HIP_CHECK(hipMalloc(&m->d_layers, table.size() * sizeof(LayerPtrs)));
-        HIP_CHECK(hipMemcpy(m->d_layers, table.data(), table.size() * sizeof(LayerPtrs),
-                            hipMemcpyHostToDevice));
-    }
     if (shape.modern()) {
         // The rotation angles of every position, with the reference's own fp32
         // expression (inference.cpp:169-175).
@@ -705,6 +695,26 @@ static const char* persist_unavailable(const Session& s, int lds_bytes, int cus)
     if (sh.max_len > 4096) return "the persistent engine handles contexts up to 4096";
     if (cus < sh.heads) return "the GPU has fewer compute units than the model has heads";
     (void)lds_bytes;
+    // The kernel finds a layer's tensors by address arithmetic (layer_at): they must
+    // follow each other without gaps, layer after layer.
+    {
+        const size_t d = sh.d_model, F = sh.d_ff();
+        const size_t per_layer = layer_floats(d, F, sh.modern());
+        const float* base = s.m->layers[0].wqkv;
+        for (size_t l = 0; l < s.m->layers.size(); l++) {
+            const LayerWeights& w = s.m->layers[l];
+            const float* b = base + l * per_layer;
+            const float* want[12];
+            size_t i = 0;
+            for (const size_t n : {3 * d * d, 3 * d, d * d, d, (sh.modern() ? 2 : 1) * F * d, F, d * F, d, d, d, d, d}) {
+                want[i++] = b;
+                b += n;
+            }
+            const float* have[12] = {w.wqkv, w.bqkv, w.wo, w.bo, w.w1, w.b1, w.w2, w.b2, w.g1, w.be1, w.g2, w.be2};
+            for (i = 0; i < 12; i++)
+                if (have[i] != want[i]) return "the persistent engine needs the layers' tensors back to back";
+        }
+    }
     return nullptr;
 }
 
@@ -732,7 +742,7 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     PersistParams p{};
     p.E = m.E;
     p.P = m.P;
-    p.layers = m.d_layers;
+    p.layer0 = m.layers[0].wqkv;
     p.gf = m.gf;
     p.bf = m.bf;
     p.rope_cos = m.rope_cos;

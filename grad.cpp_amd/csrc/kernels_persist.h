@@ -36,6 +36,38 @@ struct LayerPtrs {
     const float *wqkv, *bqkv, *wo, *bo, *w1, *b1, *w2, *b2, *g1, *be1, *g2, *be2;
 };
 
+// Floats of one layer when its tensors follow each other in the order of
+// LayerPtrs with no gaps (every size is a multiple of 64 floats when d_model
+// and the FFN width are multiples of 256): w1 holds gate and up rows for the
+// Modern block, b1 has F entries in both.
+constexpr size_t layer_floats(size_t D, size_t F, bool modern) {
+    return 3 * D * D + 3 * D + D * D + D + (modern ? 2 : 1) * F * D + F + D * F + D + 4 * D;
+}
+
+// The tensors of layer l of such a blob.  Plain address arithmetic on a kernel
+// argument: no table to fetch before the rows can be requested, and the
+// compiler knows the rows are in global memory.
+template <int KD, int KF, bool MODERN>
+__device__ __forceinline__ LayerPtrs layer_at(const float* layer0, int l) {
+    constexpr size_t D = KD * 256, F = KF * 256;
+    const float* b = layer0 + static_cast<size_t>(l) * layer_floats(D, F, MODERN);
+    asm volatile("" : "+s"(b));
+    LayerPtrs w;
+    w.wqkv = b, b += 3 * D * D;
+    w.bqkv = b, b += 3 * D;
+    w.wo = b, b += D * D;
+    w.bo = b, b += D;
+    w.w1 = b, b += (MODERN ? 2 : 1) * F * D;
+    w.b1 = b, b += F;
+    w.w2 = b, b += D * F;
+    w.b2 = b, b += D;
+    w.g1 = b, b += D;
+    w.be1 = b, b += D;
+    w.g2 = b, b += D;
+    w.be2 = b;
+    return w;
+}
+
 struct PersistCtl {
     unsigned abort;     // set by any workgroup that gave up waiting
     unsigned where;     // phase tag it was waiting for (diagnostics)
@@ -46,7 +78,7 @@ struct PersistCtl {
 struct PersistParams {
     const float* E;
     const float* P;
-    const LayerPtrs* layers;  // device array
+    const float* layer0;  // layer 0's first tensor; the layers follow each other as layer_at() says
     const float *gf, *bf, *rope_cos, *rope_sin;
     int d, F, V, L, H;
     KvLayout kv;
@@ -411,7 +443,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         // Operands of layer 0's QKV are fetched while the token arrives.
         QkvOperands<KD, PRO> qo;
         {
-            const LayerPtrs w0l = p.layers[0];
+            const LayerPtrs w0l = layer_at<KD, KF, MODERN>(p.layer0, 0);
             if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, w0l, first, pos, lane, qo);
             else qo = QkvOperands<KD, PRO>{};  // nothing to keep alive across steps
         }
@@ -440,7 +472,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         __syncthreads();
 
         for (int l = 0; l < L; l++) {
-            const LayerPtrs w = p.layers[l];
+            const LayerPtrs w = layer_at<KD, KF, MODERN>(p.layer0, l);
             // Keep the compiler from hoisting every lane- and item-derived address of
             // every phase out of the layer loop (they would not fit in registers and
             // would be spilled to scratch memory): re-derive them per layer.
@@ -754,7 +786,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             // ===== the next consumer of x is layer l+1's QKV: its operands are
             // fetched while x is still being exchanged.
             if (l + 1 < L) {
-                const LayerPtrs wn = p.layers[l + 1];
+                const LayerPtrs wn = layer_at<KD, KF, MODERN>(p.layer0, l + 1);
                 if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, wn, first, pos, lane, qo);
                 else qo = QkvOperands<KD, PRO>{};
                 __syncthreads();  // xs is overwritten next
