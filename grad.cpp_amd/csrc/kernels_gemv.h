@@ -107,8 +107,12 @@ __device__ __forceinline__ void store_qkv(const GemvParams& p, int m, int row, f
         const int hs = p.kv.head_size;
         const int head = c / hs, j = c - head * hs;
         const int slot = o.pos & ((1 << p.kv.page_shift) - 1);
+        // The page number is first touched here: widened to 64 bits where it was
+        // fetched, it would have to arrive before the kernel's main loads go out.
+        int page = o.page;
+        asm volatile("" : "+v"(page));
         const size_t run =
-            (((static_cast<size_t>(p.layer) * p.kv.n_pages + o.page) * 2 + (sec - 1)) * p.kv.heads + head);
+            (((static_cast<size_t>(p.layer) * p.kv.n_pages + page) * 2 + (sec - 1)) * p.kv.heads + head);
         p.kv.pool[((run << p.kv.page_shift) + slot) * hs + j] = v;
     }
 }
