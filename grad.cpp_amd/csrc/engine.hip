@@ -753,15 +753,7 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     p.L = sh.layers;
     p.H = sh.heads;
     p.kv = kv_layout(s);
-    const size_t d = sh.d_model;
-    p.xa = s.cells;
-    p.xb = s.cells + d;
-    p.q = s.cells + 2 * d;
-    p.kn = s.cells + 3 * d;
-    p.vn = s.cells + 4 * d;
-    p.at = s.cells + 5 * d;
-    p.hid = s.cells + 6 * d;
-    p.tokc = s.cells + 6 * d + sh.d_ff();
+    p.cells = s.cells;
     p.logits = s.logits;
     p.logit_log = logit_log;
     p.ctl = s.ctl;

@@ -82,7 +82,12 @@ struct PersistParams {
     const float *gf, *bf, *rope_cos, *rope_sin;
     int d, F, V, L, H;
     KvLayout kv;
-    Cell *xa, *xb, *q, *kn, *vn, *at, *hid, *tokc;
+    // One block of exchange cells, in this order: x after a layer [d], x after the
+    // attention half [d], q [d], new key [d], new value [d], attention output [d],
+    // FFN hidden [F], the picked token [1].  The kernel addresses them from the one
+    // base: eight pointers held through the whole token loop are sixteen scalar
+    // registers that would otherwise be parked in vector lanes and fetched back.
+    Cell* cells;
     float* logits;     // [V]
     float* logit_log;  // [steps][V] or nullptr
     PersistCtl* ctl;
@@ -211,7 +216,7 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
         const unsigned stop = __hip_atomic_load(p.stop_request, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         if (__builtin_amdgcn_readfirstlane(stop) != 0u) {
             if (tid == 0) {
-                cell_put(p.tokc, __int_as_float(-1), tok_tag);
+                cell_put((p.cells + 6 * p.d + p.F), __int_as_float(-1), tok_tag);
                 feed_put(p, i_pick, -1);
             }
             return false;
@@ -254,7 +259,7 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
                                : pick_body<true, kPersistThreads>(pk, 0, pk.work, lds, u);
     if (tid == 0) {
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        cell_put(p.tokc, __int_as_float(chosen), tok_tag);
+        cell_put((p.cells + 6 * p.d + p.F), __int_as_float(chosen), tok_tag);
         if constexpr (FEED) feed_put(p, i_pick, chosen);
         if (pp) pp[1] = __builtin_amdgcn_s_memrealtime();
     }
@@ -456,7 +461,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             // the pick that followed step s-1 (or opened the launch)
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
-            if (!gather_cells(p.tokc, 1, tt, ascr, p)) return;
+            if (!gather_cells((p.cells + 6 * D + F), 1, tt, ascr, p)) return;
             tok = __float_as_int(ascr[0]);
             __syncthreads();
             if constexpr (FEED) {
@@ -498,10 +503,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                     }
                     const unsigned t = tag_of(l, 0);
                     if (sec == 0) {
-                        cell_put(p.q + col, a, t);
-                        cell_put(p.q + col + 1, c, t);
+                        cell_put((p.cells + 2 * D) + col, a, t);
+                        cell_put((p.cells + 2 * D) + col + 1, c, t);
                     } else {
-                        Cell* dst = (sec == 1 ? p.kn : p.vn) + col;
+                        Cell* dst = (sec == 1 ? (p.cells + 3 * D) : (p.cells + 4 * D)) + col;
                         cell_put(dst, a, t);
                         cell_put(dst + 1, c, t);
                         const int head = col / HS, jj = col - head * HS;
@@ -549,7 +554,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                     bool failed = false;
                     if (tid < 96) {
                         const int seg = tid >> 5, j = (tid & 31) * 2;
-                        const Cell* src = (seg == 0 ? p.q : seg == 1 ? p.kn : p.vn) + hd * HS;
+                        const Cell* src = (seg == 0 ? (p.cells + 2 * D) : seg == 1 ? (p.cells + 3 * D) : (p.cells + 4 * D)) + hd * HS;
                         const __amdgpu_buffer_rsrc_t rs = make_buffer(src, HS * 8u);
                         for (;;) {
                             const v4i w = coherent_load16(rs, static_cast<unsigned>(j) * 8u);
@@ -665,7 +670,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                         Lsum += part[w8 * 68 + 1] * f;
                         o += part[w8 * 68 + 4 + tid] * f;
                     }
-                    cell_put(p.at + hd * HS + tid, o * (1.0f / Lsum), tag_of(l, 1));
+                    cell_put((p.cells + 5 * D) + hd * HS + tid, o * (1.0f / Lsum), tag_of(l, 1));
                 }
                 __syncthreads();
             }
@@ -714,10 +719,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
 #pragma unroll
                     for (int i = 0; i < KD; i++) w0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
-                if (!gather_cells(p.at, D, tag_of(l, 1), vin, p)) return;
+                if (!gather_cells((p.cells + 5 * D), D, tag_of(l, 1), vin, p)) return;
                 for (int row = first; row < D; ) {
                     const float a = dot_row_lds<KD>(w0, vin, lane);
-                    if (lane == 0) cell_put(p.xb + row, (xs[row] + bo) + a, tag_of(l, 2));
+                    if (lane == 0) cell_put((p.cells + D) + row, (xs[row] + bo) + a, tag_of(l, 2));
                     row += stride;
                     if (row < D) {
                         load_row<KD>(w.wo, row, D, lane, w0);
@@ -731,7 +736,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             {
                 if (!early_ffn1) load_ffn1();
                 __syncthreads();  // every wave is done reading xs (phase C)
-                if (!gather_cells(p.xb, D, tag_of(l, 2), xs, p)) return;
+                if (!gather_cells((p.cells + D), D, tag_of(l, 2), xs, p)) return;
                 for (int item = first; item < NIT; ) {
                     float4 h[KD];
                     load_input<KD, PRO>(xs, n2, lane, h);
@@ -740,10 +745,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                     if (lane == 0) {
                         const unsigned t = tag_of(l, 3);
                         if (MODERN) {
-                            cell_put(p.hid + item, c * silu(a), t);
+                            cell_put((p.cells + 6 * D) + item, c * silu(a), t);
                         } else {
-                            cell_put(p.hid + 2 * item, gelu_tanh(a + fb0), t);
-                            cell_put(p.hid + 2 * item + 1, gelu_tanh(c + fb1), t);
+                            cell_put((p.cells + 6 * D) + 2 * item, gelu_tanh(a + fb0), t);
+                            cell_put((p.cells + 6 * D) + 2 * item + 1, gelu_tanh(c + fb1), t);
                         }
                     }
                     item += stride;
@@ -770,10 +775,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
 #pragma unroll
                     for (int i = 0; i < KF; i++) w0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
-                if (!gather_cells(p.hid, F, tag_of(l, 3), vin, p)) return;
+                if (!gather_cells((p.cells + 6 * D), F, tag_of(l, 3), vin, p)) return;
                 for (int row = first; row < D; ) {
                     const float a = dot_row_lds<KF>(w0, vin, lane);
-                    if (lane == 0) cell_put(p.xa + row, (xs[row] + b2) + a, tag_of(l, 4));
+                    if (lane == 0) cell_put(p.cells + row, (xs[row] + b2) + a, tag_of(l, 4));
                     row += stride;
                     if (row < D) {
                         load_row<KF>(w.w2, row, F, lane, w0);
@@ -790,7 +795,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, wn, first, pos, lane, qo);
                 else qo = QkvOperands<KD, PRO>{};
                 __syncthreads();  // xs is overwritten next
-                if (!gather_cells(p.xa, D, tag_of(l, 4), xs, p)) return;
+                if (!gather_cells(p.cells, D, tag_of(l, 4), xs, p)) return;
             }
         }
 
@@ -806,7 +811,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
 #pragma unroll
             for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(first * RL + r, V - 1), D, lane, wr[r]);
             __syncthreads();
-            if (!gather_cells(p.xa, D, tag_of(L - 1, 4), xs, p)) return;
+            if (!gather_cells(p.cells, D, tag_of(L - 1, 4), xs, p)) return;
             stamp();
             float4 h[KD];
             load_input<KD, PRO>(xs, nf, lane, h);
