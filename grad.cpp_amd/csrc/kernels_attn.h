@@ -281,20 +281,30 @@ __global__ __launch_bounds__(256) void attn_decode64_kernel(const AttnParams p) 
         mb = fmaxf(mb, dpp_move<0x143, 0xC>(mb, mb));
         mb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mb), 63));
         const float mn = fmaxf(m, mb);
-        const float f = expf(m - mn);  // 0 on the first batch
+        // The 16 lanes of a position group hold the same eight scores and the same
+        // running maximum: lane dl forms one exponential, that of score dl (lane 8:
+        // of the old maximum, the rescaling factor), and the group shares them by row
+        // broadcasts, one exponential per lane and batch instead of nine.
+        float arg = sc[0];
+#pragma unroll
+        for (int it = 1; it < 8; it++) arg = (dl == it) ? sc[it] : arg;
+        arg = (dl == 8) ? m : arg;
+        const float em = expf(arg - mn);  // exp(-inf) = 0: past the end of the run, first batch
+        const float f = row_lane<8>(em);
         lsum *= f;
         acc.x *= f;
         acc.y *= f;
         acc.z *= f;
         acc.w *= f;
+        const float e[8] = {row_lane<0>(em), row_lane<1>(em), row_lane<2>(em), row_lane<3>(em),
+                            row_lane<4>(em), row_lane<5>(em), row_lane<6>(em), row_lane<7>(em)};
 #pragma unroll
         for (int it = 0; it < 8; it++) {
-            const float e = expf(sc[it] - mn);  // exp(-inf) = 0 past the end of the run
-            lsum += e;
-            acc.x += e * v4[it].x;
-            acc.y += e * v4[it].y;
-            acc.z += e * v4[it].z;
-            acc.w += e * v4[it].w;
+            lsum += e[it];
+            acc.x += e[it] * v4[it].x;
+            acc.y += e[it] * v4[it].y;
+            acc.z += e[it] * v4[it].z;
+            acc.w += e[it] * v4[it].w;
         }
         m = mn;
     }

@@ -88,6 +88,13 @@ __device__ __forceinline__ float wave_max(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Lane N of every row of 16 lanes, handed to all lanes of that row.
+template <int N>
+__device__ __forceinline__ float row_lane(float v) {
+    static_assert(N >= 0 && N < 16, "a row has 16 lanes");
+    return dpp_move<0x150 + N, 0xF>(v, 0.0f);  // row_newbcast:N
+}
+
 // Block-wide reductions through a small LDS scratch (one float per wave).
 // Every thread of the block must call them; all threads get the result.
 // nt: threads of the workgroup; a caller that knows it at compile time passes it

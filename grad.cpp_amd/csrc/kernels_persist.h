@@ -619,20 +619,31 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                     mb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mb), 63));
                     const float mn = fmaxf(m, mb);
                     if (mn > -INFINITY) {
-                        const float f = expf(m - mn);  // 0 on the first batch (m = -inf)
+                        // The 16 lanes of a position group hold the same eight scores and the
+                        // same running maximum.  Lane dl forms one exponential, that of score
+                        // dl (lane 8: of the old maximum, the rescaling factor), and the group
+                        // shares them by row broadcasts: one exponential per lane and batch
+                        // instead of nine, with the same values.
+                        float arg = sc[0];
+#pragma unroll
+                        for (int it = 1; it < 8; it++) arg = (dl == it) ? sc[it] : arg;
+                        arg = (dl == 8) ? m : arg;
+                        const float em = expf(arg - mn);  // exp(-inf) = 0: unused slots, first batch
+                        const float f = row_lane<8>(em);
                         lsum *= f;
                         acc.x *= f;
                         acc.y *= f;
                         acc.z *= f;
                         acc.w *= f;
+                        const float e[8] = {row_lane<0>(em), row_lane<1>(em), row_lane<2>(em), row_lane<3>(em),
+                                            row_lane<4>(em), row_lane<5>(em), row_lane<6>(em), row_lane<7>(em)};
 #pragma unroll
                         for (int it = 0; it < 8; it++) {
-                            const float e = expf(sc[it] - mn);  // exp(-inf) = 0 for unused slots
-                            lsum += e;
-                            acc.x += e * v4[it].x;
-                            acc.y += e * v4[it].y;
-                            acc.z += e * v4[it].z;
-                            acc.w += e * v4[it].w;
+                            lsum += e[it];
+                            acc.x += e[it] * v4[it].x;
+                            acc.y += e[it] * v4[it].y;
+                            acc.z += e[it] * v4[it].z;
+                            acc.w += e[it] * v4[it].w;
                         }
                         m = mn;
                     }
@@ -664,9 +675,12 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
 #pragma unroll
                     for (int w8 = 0; w8 < kPersistWaves; w8++) M = fmaxf(M, part[w8 * 68]);
                     float Lsum = 0.0f, o = 0.0f;
+                    // one exponential per lane (wavefront lane % 8's), read across by all
+                    static_assert(kPersistWaves == 8, "lane % 8 picks a wavefront");
+                    const float fmine = expf(part[(tid & 7) * 68] - M);  // 0 for wavefronts without positions
 #pragma unroll
                     for (int w8 = 0; w8 < kPersistWaves; w8++) {
-                        const float f = expf(part[w8 * 68] - M);  // 0 for wavefronts without positions
+                        const float f = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fmine), w8));
                         Lsum += part[w8 * 68 + 1] * f;
                         o += part[w8 * 68 + 4 + tid] * f;
                     }
