@@ -88,6 +88,23 @@ __device__ __forceinline__ float wave_max(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Running total over the lanes of a wavefront, this lane's own value included:
+// shifts inside each row of 16, then the totals of the rows before.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_move_int(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xF, false);  // lanes without a source get 0
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+    v += dpp_move_int<0x111, 0xF>(v);  // row_shr:1
+    v += dpp_move_int<0x112, 0xF>(v);  // row_shr:2
+    v += dpp_move_int<0x114, 0xF>(v);  // row_shr:4
+    v += dpp_move_int<0x118, 0xF>(v);  // row_shr:8
+    v += dpp_move_int<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_move_int<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 // Lane N of every row of 16 lanes, handed to all lanes of that row.
 template <int N>
 __device__ __forceinline__ float row_lane(float v) {

@@ -419,8 +419,17 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
     unsigned long long mine = 0ull;
 #pragma unroll
     for (int r = 0; r < ROUNDS; r++) mine |= static_cast<unsigned long long>(x[r] >= T) << r;
+    // slots: one atomic per wavefront (a running count over its lanes), not one per thread
+    const int mine_n = __popcll(mine);
+    const int upto = wave_inclusive_scan(mine_n);
+    const int wave_n = __builtin_amdgcn_readlane(upto, 63);
+    int wave_base = 0;
+    if (wave_n) {  // uniform
+        if (lane == 63) wave_base = atomicAdd(&ishare[1], wave_n);
+        wave_base = __builtin_amdgcn_readlane(wave_base, 63);
+    }
     if (mine) {
-        int slot = atomicAdd(&ishare[1], __popcll(mine));
+        int slot = wave_base + upto - mine_n;
         while (mine) {
             const int r = __ffsll(static_cast<long long>(mine)) - 1;
             mine &= mine - 1ull;
