@@ -343,6 +343,38 @@ __device__ __forceinline__ float wave_total_in_order(float x, int n) {
     return acc;
 }
 
+// The same two walks over a list that sits in LDS (n a multiple of 8, the list
+// padded with zeros): every lane reads every element (one address per read, a
+// broadcast) and runs the chain of additions itself.  Same order of additions,
+// same results; no lane-to-scalar move in front of each one.
+__device__ __forceinline__ float lds_total_in_order(const float* x, int n) {
+    float acc = 0.0f;
+    for (int j = 0; j < n; j += 8) {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) v[q] = x[j + q];
+#pragma unroll
+        for (int q = 0; q < 8; q++) acc += v[q];
+    }
+    return acc;
+}
+
+__device__ __forceinline__ int lds_prefixes_below(const float* x, int n, float thr) {
+    float acc = 0.0f;
+    int below = 0;
+    for (int j = 0; j < n; j += 8) {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) v[q] = x[j + q];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            acc += v[q];
+            below += (acc < thr) ? 1 : 0;
+        }
+    }
+    return below;
+}
+
 constexpr int kFastCandCap = 512;
 // LDS floats the fast sampler needs: candidate values, indices and ranks, the
 // survivors (value, index, index rank) and a permutation area.
@@ -492,40 +524,46 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         const float v = sv[lane];
         const int ri = live ? ridx[lane] : lane;
         const float e = live ? expf(v - sv[0]) : 0.0f;
+        float* in_order = reinterpret_cast<float*>(perm);  // [64] a value per survivor, index order
+        float* walk = cand_v;                               // [64] the list an ordered walk goes over
         // index-order copies of e and of the token ids
         perm[lane] = 0;
         perm[64 + lane] = 0x7FFFFFFF;
         __builtin_amdgcn_wave_barrier();
         if (live) {
-            perm[ri] = __float_as_int(e);
+            in_order[ri] = e;
             perm[64 + ri] = si[lane];
         }
         __builtin_amdgcn_wave_barrier();
-        const float eo = __int_as_float(perm[lane]);
-        const int io = perm[64 + lane];
-        __builtin_amdgcn_wave_barrier();
-        const float inv_sum = 1.0f / wave_total_in_order(eo, n);
+        const float eo = in_order[lane];
+        const float inv_sum = 1.0f / lds_total_in_order(in_order, n);
         float po = eo * inv_sum;  // index order
         if (top_p < 1.0f) {
             float pr = e * inv_sum;  // descending order
+            walk[lane] = pr;
+            __builtin_amdgcn_wave_barrier();
             // first position whose running sum reaches top_p; never reached: only the
             // maximum survives
-            const int reach = wave_prefixes_below(pr, n, top_p);
+            const int reach = lds_prefixes_below(walk, n, top_p);
             const int at = reach < S ? reach : 0;
-            const float cutoff = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pr), at));
+            const float cutoff = walk[at];
             if (!(live && pr > 0.0f && pr >= cutoff)) pr = 0.0f;
-            perm[lane] = 0;
             __builtin_amdgcn_wave_barrier();
-            if (live) perm[ri] = __float_as_int(pr);
+            in_order[lane] = 0.0f;
             __builtin_amdgcn_wave_barrier();
-            po = __int_as_float(perm[lane]);
-            const float total = wave_total_in_order(po, n);
+            if (live) in_order[ri] = pr;
+            __builtin_amdgcn_wave_barrier();
+            po = in_order[lane];
+            const float total = lds_total_in_order(in_order, n);
             if (total > 0.0f) po = po / total;
         }
         int chosen = 0;
         if (u > 0.0f) {
-            const int hit = wave_prefixes_below(po, n, u);  // first i with u <= cumulative
-            chosen = hit < S ? __builtin_amdgcn_readlane(io, hit) : V - 1;
+            __builtin_amdgcn_wave_barrier();
+            walk[lane] = po;
+            __builtin_amdgcn_wave_barrier();
+            const int hit = lds_prefixes_below(walk, n, u);  // first i with u <= cumulative
+            chosen = hit < S ? perm[64 + hit] : V - 1;
         }
         if (tid == 0) ishare[1] = chosen;
     }
