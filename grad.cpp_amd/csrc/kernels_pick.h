@@ -738,8 +738,6 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
     __shared__ int redi[kPickThreads / 64];
     __shared__ unsigned hist256[256];
     __shared__ unsigned bcast[2];
-    __shared__ int win_tok[kPenaltyWindow];
-    __shared__ int pen_before[64], pen_count[64];
     __shared__ int ishare[2];
 
     constexpr int nt = NT;
@@ -759,13 +757,32 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
         const int* hp = &hist[p.n_hist - window + tid];
         window_token = coherent ? __hip_atomic_load(hp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *hp;
     }
+    // How often each entry of the window occurs, and whether it is the first of its
+    // kind (that one applies the penalty, once per occurrence): wavefront 0 holds the
+    // window one entry per lane and compares in registers, while the row is on its way.
+    int pen_first = 0, pen_times = 0;
+    auto count_window = [&]() {
+        if (p.penalty != 1.0f && tid < 64) {
+            const int id = tid < window ? window_token : -1 - tid;
+            int before = 0;
+            for (int e = 0; e < window; e++) {
+                const int other = __builtin_amdgcn_readlane(id, e);
+                before += (e < tid && other == id) ? 1 : 0;
+                pen_times += (other == id) ? 1 : 0;
+            }
+            pen_first = (tid < window && before == 0) ? 1 : 0;
+        }
+    };
     if (coherent) {
         const __amdgpu_buffer_rsrc_t rs = make_buffer(logits, static_cast<unsigned>(V) * 4u);
         // eight 16-byte loads per thread in flight; reads past the end return zero
+        bool counted = false;
         for (int base = 4 * tid; base < V; base += 32 * nt) {
             v4i w[8];
 #pragma unroll
             for (int q = 0; q < 8; q++) w[q] = coherent_load16(rs, static_cast<unsigned>(base + q * 4 * nt) * 4u);
+            if (!counted) count_window();
+            counted = true;
 #pragma unroll
             for (int q = 0; q < 8; q++) {
                 const int i = base + q * 4 * nt;
@@ -780,39 +797,17 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
                 }
             }
         }
+        if (!counted) count_window();
     } else {
         row_pass(logits, V, [&](int i, float v) { val[i] = v; }, nt);
-    }
-    if (tid < window) win_tok[tid] = window_token;
-    if (tid < 64) {
-        pen_before[tid] = 0;
-        pen_count[tid] = 0;
+        count_window();
     }
     __syncthreads();
     if (p.penalty != 1.0f) {
-        // Entry e of the window is handled by its first occurrence, which applies
-        // the penalty once per occurrence.  Every wavefront compares all entries
-        // with one slice of the window.
-        const int lane = tid & 63, nw = nt >> 6, wave = tid >> 6;
-        const int slice = (window + nw - 1) / nw;
-        const int j0 = wave * slice, j1 = min(window, j0 + slice);
-        const int id = lane < window ? win_tok[lane] : -1 - lane;
-        int before = 0, count = 0;
-        for (int e = j0; e < j1; e++) {
-            const int other = win_tok[e];
-            before += (e < lane && other == id);
-            count += (other == id);
-        }
-        if (lane < window && count) {
-            if (before) atomicAdd(&pen_before[lane], before);
-            atomicAdd(&pen_count[lane], count);
-        }
-        __syncthreads();
-        if (tid < window && pen_before[tid] == 0) {
-            const int tok = win_tok[tid], count_all = pen_count[tid];
-            float v = val[tok];
-            for (int c = 0; c < count_all; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
-            val[tok] = v;
+        if (pen_first) {
+            float v = val[window_token];
+            for (int c = 0; c < pen_times; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
+            val[window_token] = v;
         }
         __syncthreads();
     }

@@ -108,7 +108,9 @@ def test_prompts_around_the_one_pass_threshold(llama768, plen):
 
 def test_sessions_and_models_give_their_memory_back(llama768):
     import ctypes
-    hip = ctypes.CDLL("libamdhip64.so")
+    # by soname: the HIP runtime the process already has (the library's, or torch's when
+    # torch came first); any other name can bring a second runtime in, which finds no GPU
+    hip = ctypes.CDLL("libamdhip64.so.7")
 
     def free_bytes():
         free, total = ctypes.c_size_t(), ctypes.c_size_t()

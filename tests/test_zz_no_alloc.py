@@ -10,6 +10,17 @@ from gradhip import synth
 
 pytestmark = pytest.mark.gpu
 
+
+def _torch_on_the_loaded_runtime():
+    """torch, sharing the HIP runtime the library has brought up.  torch ships a copy of
+    the runtime and asks the loader for it as "libamdhip64.so"; a second runtime in one
+    process finds no GPU.  Loading that name first makes the loader hand torch the file
+    that is already mapped (the library links the same file under its soname)."""
+    import ctypes
+    G.device_info()  # the documented set-up call; loads the library and its runtime
+    ctypes.CDLL("libamdhip64.so")
+    return pytest.importorskip("torch")
+
 OPTIONS = [
     dict(greedy=True, repetition_penalty=1.3),
     dict(temperature=0.8, top_k=40, top_p=0.9, repetition_penalty=1.1),
@@ -45,7 +56,7 @@ def _run(torch, dev, batch, vocab, plen):
 
 
 def test_noalloc_pick_equals_session_pick_twice_in_a_row():
-    torch = pytest.importorskip("torch")
+    torch = _torch_on_the_loaded_runtime()
     G.device_info()  # the documented set-up call: looks the scratch array up on this device
     big = _case(torch, synth.Config(synth.ARCH_MODERN, 50257, 128, 2, 2, 32), 900, 3, 12)
     small = _case(torch, synth.Config(synth.ARCH_GPT2, 777, 128, 2, 2, 32), 910, 1, 9)
@@ -61,7 +72,7 @@ def test_noalloc_pick_equals_session_pick_twice_in_a_row():
 
 
 def test_noalloc_pick_philox_draws_and_limits():
-    torch = pytest.importorskip("torch")
+    torch = _torch_on_the_loaded_runtime()
     cfg = synth.Config(synth.ARCH_MODERN, 1000, 128, 2, 2, 32)
     W = synth.make_weights(cfg, 920, std=0.08)
     gs = G.Session(G.Model.from_tensors(cfg, W))
