@@ -64,6 +64,16 @@ template <int EPI, bool RMS, int MT, int NT, int KW>
 __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int M, int m_groups) {
     __shared__ float red[KW][MT][NT][16 * 16];
     __shared__ float ssq[KW][MT][16];
+    // Every scalar argument the kernel reads is named here, at its start: the
+    // compiler fetches an argument in the block that first uses it, and with the
+    // uses spread behind the early exit and the epilogue's conditions that made four
+    // fetches from the argument segment, each waited for before the next, in front
+    // of the first weight load.  Named together they are one batch and one wait.
+    asm volatile("" ::"s"(p.W), "s"(p.in), "s"(p.out), "s"(p.bias), "s"(p.gamma), "s"(p.N), "s"(p.K),
+                 "s"(p.in_stride), "s"(p.out_stride), "s"(M), "s"(m_groups));
+    if constexpr (EPI == EPI_QKV)
+        asm volatile("" ::"s"(p.st), "s"(p.rope_cos), "s"(p.rope_sin), "s"(p.kv.page_table), "s"(p.kv.pool),
+                     "s"(p.d_model), "s"(p.rows_per_seq), "s"(p.kv.pages_per_seq), "s"(p.kv.page_shift));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // id -> (weight group, row group): ids with the same id % 8 and consecutive id / 8 share weights
     const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
