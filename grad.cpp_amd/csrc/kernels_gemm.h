@@ -140,27 +140,43 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
     // 0.568 -> 0.553 ms; two, three, five and six were all slower than four).
     constexpr int UNROLL = (MT + NT + 1) <= 6 ? 4 : 2;
 
-    auto consume = [&](const float4 (&a_in)[MT], const float4 (&b_in)[NT], const float4& g4) {
-        float4 as[MT], b[NT];
+    // One K-step in two halves.  prepare(): the fetched float4s go to the lanes that feed
+    // them to the matrix core (ds_bpermute, a trip through the LDS crossbar each), with
+    // the norm's share of the work.  multiply(): the products.  The halves of
+    // neighbouring steps are interleaved below, the permutes of step u + 1 going out
+    // before the products of step u, so that the crossbar's latency is paid beside the
+    // products instead of in front of every one of them; sched_barrier keeps the
+    // compiler from folding the two back into permute, wait, multiply, permute, ...
+    // Only for one tile per workgroup: with more tiles (64 rows against wide
+    // projections) the operands held for two steps cost registers and occupancy, and a
+    // step measured slower that way (c3 421.5 -> 434.8 us; c4, all 1 x 1, 547.7 -> 544.8).
+    constexpr bool kInterleave = MT * NT == 1;
+    struct Operands {
+        float4 a[MT], b[NT];
+    };
+    auto prepare = [&](const float4 (&a_in)[MT], const float4 (&b_in)[NT], const float4& g4, Operands& o) {
 #pragma unroll
-        for (int u = 0; u < NT; u++) b[u] = to_operand(b_in[u]);
+        for (int u = 0; u < NT; u++) o.b[u] = to_operand(b_in[u]);
 #pragma unroll
-        for (int t = 0; t < MT; t++) {
-            const float4 a = to_operand(a_in[t]);
-            as[t] = a;
-            if (RMS) {
+        for (int t = 0; t < MT; t++) o.a[t] = to_operand(a_in[t]);
+        if (RMS) {
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                const float4 a = o.a[t];
                 ss[t] += dot4(a, a);
-                as[t] = make_float4(a.x * g4.x, a.y * g4.y, a.z * g4.z, a.w * g4.w);
+                o.a[t] = make_float4(a.x * g4.x, a.y * g4.y, a.z * g4.z, a.w * g4.w);
             }
         }
+    };
+    auto multiply = [&](const Operands& o) {
 #pragma unroll
         for (int t = 0; t < MT; t++)
 #pragma unroll
             for (int u = 0; u < NT; u++) {
-                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].x, b[u].x, acc[t][u], 0, 0, 0);
-                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].y, b[u].y, acc[t][u], 0, 0, 0);
-                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].z, b[u].z, acc[t][u], 0, 0, 0);
-                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(as[t].w, b[u].w, acc[t][u], 0, 0, 0);
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[t].x, o.b[u].x, acc[t][u], 0, 0, 0);
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[t].y, o.b[u].y, acc[t][u], 0, 0, 0);
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[t].z, o.b[u].z, acc[t][u], 0, 0, 0);
+                acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[t].w, o.b[u].w, acc[t][u], 0, 0, 0);
             }
     };
     int k = 0;
@@ -174,8 +190,24 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
             for (int t = 0; t < MT; t++) a[u][t] = *reinterpret_cast<const float4*>(ap[t] + k + 16 * u);
             gm[u] = RMS ? *reinterpret_cast<const float4*>(gp + k + 16 * u) : make_float4(1.f, 1.f, 1.f, 1.f);
         }
+        if constexpr (kInterleave) {
+            Operands o[2];
+            prepare(a[0], b[0], gm[0], o[0]);
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) consume(a[u], b[u], gm[u]);
+            for (int u = 0; u < UNROLL; u++) {
+                if (u + 1 < UNROLL) prepare(a[u + 1], b[u + 1], gm[u + 1], o[(u + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                multiply(o[u & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                Operands o;
+                prepare(a[u], b[u], gm[u], o);
+                multiply(o);
+            }
+        }
     }
     if (k < kq) {
         // The steps left over go out as one more round with every load in flight: a
@@ -192,7 +224,11 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
         }
 #pragma unroll
         for (int u = 0; u < UNROLL - 1; u++)
-            if (k + 16 * u < kq) consume(a[u], b[u], gm[u]);
+            if (k + 16 * u < kq) {
+                Operands o;
+                prepare(a[u], b[u], gm[u], o);
+                multiply(o);
+            }
     }
     // Accumulator layout: lane holds column j, rows 4*g + r.
 #pragma unroll
