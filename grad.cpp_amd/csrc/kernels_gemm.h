@@ -222,13 +222,24 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
             for (int t = 0; t < MT; t++) a[u][t] = *reinterpret_cast<const float4*>(ap[t] + kk);
             gm[u] = RMS ? *reinterpret_cast<const float4*>(gp + kk) : make_float4(1.f, 1.f, 1.f, 1.f);
         }
+        if constexpr (kInterleave) {
+            Operands o[UNROLL - 1];
 #pragma unroll
-        for (int u = 0; u < UNROLL - 1; u++)
-            if (k + 16 * u < kq) {
-                Operands o;
-                prepare(a[u], b[u], gm[u], o);
-                multiply(o);
-            }
+            for (int u = 0; u < UNROLL - 1; u++)
+                if (k + 16 * u < kq) prepare(a[u], b[u], gm[u], o[u]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < UNROLL - 1; u++)
+                if (k + 16 * u < kq) multiply(o[u]);
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNROLL - 1; u++)
+                if (k + 16 * u < kq) {
+                    Operands o;
+                    prepare(a[u], b[u], gm[u], o);
+                    multiply(o);
+                }
+        }
     }
     // Accumulator layout: lane holds column j, rows 4*g + r.
 #pragma unroll
