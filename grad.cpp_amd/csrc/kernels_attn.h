@@ -48,19 +48,53 @@ __device__ __forceinline__ bool last_chunk_arrived(unsigned* ticket_ctr, int nch
 __device__ __forceinline__ void attn_merge(const AttnParams& p, int b, int h, int nchunk, int hs) {
     const float* base = p.part + (static_cast<size_t>(b) * p.kv.heads + h) * p.max_chunks * (hs + 2);
     const __amdgpu_buffer_rsrc_t rs = make_buffer(base, static_cast<unsigned>(nchunk * (hs + 2)) * 4u);
-    auto at = [&](int i) {  // one float through a device-scope load
-        const v4i w = coherent_load16(rs, static_cast<unsigned>(i & ~3) * 4u);
-        return __int_as_float(w[i & 3]);
-    };
+    // Element i of the partials through a device-scope load of the 16 bytes around it.
+    // The loads of four chunks go out together: one after the other, each waited for,
+    // they were three dependent trips to memory per chunk at the very end of the launch,
+    // where nothing else is left to hide them.
+    auto fetch = [&](int i) { return coherent_load16(rs, static_cast<unsigned>(i & ~3) * 4u); };
+    auto pick = [](const v4i& w, int i) { return __int_as_float(w[i & 3]); };
+    const int stride = hs + 2;
     float M = -INFINITY;
-    for (int s = 0; s < nchunk; s++) M = fmaxf(M, at(s * (hs + 2)));
-    float L = 0.0f;
-    for (int s = 0; s < nchunk; s++) L += at(s * (hs + 2) + 1) * expf(at(s * (hs + 2)) - M);
+    for (int s0 = 0; s0 < nchunk; s0 += 4) {
+        v4i w[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) w[q] = fetch(min(s0 + q, nchunk - 1) * stride);
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (s0 + q < nchunk) M = fmaxf(M, pick(w[q], (s0 + q) * stride));
+    }
+    // every thread forms L (the same additions in the same order); thread j < hs forms output j
+    const int tid = threadIdx.x;
+    const int jj = tid < hs ? tid : 0;
+    float L = 0.0f, o = 0.0f;
+    for (int s0 = 0; s0 < nchunk; s0 += 4) {
+        v4i wm[4], wl[4], wa[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int at = min(s0 + q, nchunk - 1) * stride;
+            wm[q] = fetch(at);
+            wl[q] = fetch(at + 1);
+            wa[q] = fetch(at + 2 + jj);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if (s0 + q < nchunk) {
+                const int at = (s0 + q) * stride;
+                const float f = expf(pick(wm[q], at) - M);
+                L += pick(wl[q], at + 1) * f;
+                o += pick(wa[q], at + 2 + jj) * f;
+            }
+        }
+    }
     const float inv = 1.0f / L;
-    for (int j = threadIdx.x; j < hs; j += blockDim.x) {
-        float o = 0.0f;
-        for (int s = 0; s < nchunk; s++) o += at(s * (hs + 2) + 2 + j) * expf(at(s * (hs + 2)) - M);
-        p.out[static_cast<size_t>(b) * p.d_model + h * hs + j] = o * inv;
+    if (tid < hs) p.out[static_cast<size_t>(b) * p.d_model + h * hs + tid] = o * inv;
+    // head sizes beyond the workgroup (none of the shapes in use): the remaining outputs, one at a time
+    for (int j = tid + blockDim.x; j < hs; j += blockDim.x) {
+        float oj = 0.0f;
+        for (int s = 0; s < nchunk; s++)
+            oj += pick(fetch(s * stride + 2 + j), s * stride + 2 + j) * expf(pick(fetch(s * stride), s * stride) - M);
+        p.out[static_cast<size_t>(b) * p.d_model + h * hs + j] = oj * inv;
     }
 }
 
