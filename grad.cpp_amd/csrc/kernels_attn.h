@@ -55,6 +55,37 @@ __device__ __forceinline__ void attn_merge(const AttnParams& p, int b, int h, in
     auto fetch = [&](int i) { return coherent_load16(rs, static_cast<unsigned>(i & ~3) * 4u); };
     auto pick = [](const v4i& w, int i) { return __int_as_float(w[i & 3]); };
     const int stride = hs + 2;
+    if (nchunk <= 4) {
+        // everything in one round of loads
+        const int tid = threadIdx.x;
+        const int jj = tid < hs ? tid : 0;
+        v4i wm[4], wl[4], wa[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int at = min(q, nchunk - 1) * stride;
+            wm[q] = fetch(at);
+            wl[q] = fetch(at + 1);
+            wa[q] = fetch(at + 2 + jj);
+        }
+        float M = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (q < nchunk) M = fmaxf(M, pick(wm[q], q * stride));
+        float L = 0.0f, o = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if (q < nchunk) {
+                const float f = expf(pick(wm[q], q * stride) - M);
+                L += pick(wl[q], q * stride + 1) * f;
+                o += pick(wa[q], q * stride + 2 + jj) * f;
+            }
+        }
+        if (tid < hs && hs <= static_cast<int>(blockDim.x)) {
+            p.out[static_cast<size_t>(b) * p.d_model + h * hs + tid] = o * (1.0f / L);
+            return;
+        }
+        if (hs <= static_cast<int>(blockDim.x)) return;
+    }
     float M = -INFINITY;
     for (int s0 = 0; s0 < nchunk; s0 += 4) {
         v4i w[4];
