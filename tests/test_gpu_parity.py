@@ -98,6 +98,25 @@ def test_attention_split_over_workgroups_merges_to_the_same_logits(tiny_models, 
             assert_logits_close(got[b], one[b], 2e-5, f"{name} split vs whole, step {t}")
 
 
+@pytest.mark.parametrize("arch", [synth.ARCH_GPT2, synth.ARCH_MODERN])
+def test_attention_merges_more_than_four_chunks(arch):
+    """The merge fetches the partial results of four chunks at a time; up to four go through
+    a single round, more through two passes.  A context of 112 in runs of 16 positions walks
+    through one to seven chunks per head, ragged and full."""
+    cfg = synth.Config(arch, 211, 128, 2, 2, 112)
+    W, om = make_pair(cfg, 31, std=lively_std(cfg), norm_noise=0.1)
+    gm = G.Model.from_tensors(cfg, W)
+    gs = G.Session(gm, batch=2, flags=G.FLAG_SMALL_ATTENTION_CHUNKS, page_tokens=8, shuffle_pages=True)
+    whole = G.Session(gm, batch=2)
+    toks = synth.uniform_tokens(2 * cfg.max_len, cfg.vocab, 13).reshape(2, cfg.max_len)
+    oss = [O.Session(om) for _ in range(2)]
+    for t in range(cfg.max_len):
+        got, one = gs.step(toks[:, t]), whole.step(toks[:, t])
+        for b in range(2):
+            assert_logits_close(got[b], oss[b].step(toks[b, t]), TOL, f"seven chunks, arch {arch} seq {b} step {t}")
+            assert_logits_close(got[b], one[b], 2e-5, f"seven chunks vs whole, arch {arch} step {t}")
+
+
 @pytest.mark.parametrize("name", ["hs64-gpt2", "hs64-modern"])
 @pytest.mark.parametrize("batch", [1, 3])
 def test_prompt_pass_equals_steps(tiny_models, name, batch):
