@@ -84,7 +84,16 @@ __device__ __forceinline__ void row_pass(const float* v, int n, F f, int nt = bl
 #pragma unroll
         for (int q = 0; q < 8; q++) f(i + q * nt, x[q]);
     }
-    for (; i < n; i += nt) f(i, v[i]);
+    if (i < n) {
+        // what is left (fewer than eight elements per thread) goes out as one more round
+        // at clamped offsets: one at a time it was up to seven dependent trips to memory
+        float x[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) x[q] = v[min(i + q * nt, n - 1)];
+#pragma unroll
+        for (int q = 0; q < 8; q++)
+            if (i + q * nt < n) f(i + q * nt, x[q]);
+    }
 }
 
 // f(i, get(i)) for i = lo .. hi - 1 in that order, the values fetched eight at a
