@@ -719,6 +719,34 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             };
             const bool early_ffn1 = wave >= (D + G - 1) / G && wg >= H;
             if (early_ffn1) load_ffn1();
+            // With FFN2 rows of more than 8 KB (hidden widths above 2048) the same idle
+            // wavefronts also bring the FFN2 rows of this workgroup's first three wavefronts
+            // into this XCD's L2 (one float per 128-byte line touches a whole row), and those
+            // of a workgroup with a head on the same XCD, which has no idle time of its own:
+            // the rows are then a trip to the L2, not to HBM, when the FFN2 phase asks for
+            // them two exchanges later.  Measured on one box, us per token: hidden 3072
+            // (d768 GPT-2) 131.9 -> 124.7; at hidden 2048 it does not pay (Modern d768
+            // 115.9 -> 117.7, GPT-2 d512 77.6 -> 77.5), so those shapes go without.
+            if constexpr (F > 2048) {
+                if (early_ffn1 && wave < 2 * ((D + G - 1) / G)) {
+                    const int w3 = wave - (D + G - 1) / G;  // the wavefront whose row this one touches
+                    const int row = wg + G * w3;
+                    float touched = 0.0f;
+                    if (row < D) {
+                        touched += w.w2[static_cast<size_t>(row) * F + lane * 32];
+                        touched += w.w2[static_cast<size_t>(row) * F + (2048 + lane * 32) % F];
+                    }
+                    const int other = wg - 16;  // same XCD (workgroups go round-robin over 8)
+                    if (other >= 0 && other < H) {
+                        const int row2 = other + G * w3;
+                        if (row2 < D) {
+                            touched += w.w2[static_cast<size_t>(row2) * F + lane * 32];
+                            touched += w.w2[static_cast<size_t>(row2) * F + (2048 + lane * 32) % F];
+                        }
+                    }
+                    asm volatile("" ::"v"(touched));
+                }
+            }
 
             // ===== phase C: x += b_o + attn @ W_o
             {
