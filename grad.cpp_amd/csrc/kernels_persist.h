@@ -727,6 +727,45 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             // them two exchanges later.  Measured on one box, us per token: hidden 3072
             // (d768 GPT-2) 131.9 -> 124.7; at hidden 2048 it does not pay (Modern d768
             // 115.9 -> 117.7, GPT-2 d512 77.6 -> 77.5), so those shapes go without.
+            // A workgroup with a head comes out of the attention phase last and then has its
+            // W_o, FFN1 and FFN2 rows still to fetch from HBM, while every other workgroup
+            // waits for its outputs.  The workgroup 16 places further on (same XCD: workgroups
+            // go round-robin over 8) spends the attention phase idle; its wavefronts without a
+            // W_o row touch one float per 128-byte line of those rows, which brings them into
+            // the L2 the head workgroup will ask.  Measured on one box, us per token: Modern
+            // d768 119.4 -> 118.0, GPT-2 d512 77.6 -> 76.6; with a hidden width of 3072 the
+            // helpers' own polls come too late behind all this and a token took 9.6 us longer,
+            // so wide shapes only get the touch below.
+            if (F <= 2048 && early_ffn1 && wg - 16 >= 0 && wg - 16 < H) {
+                const int other = wg - 16;
+                const int hw = wave - (D + G - 1) / G;  // 0 .. 4
+                float touched = 0.0f;
+                constexpr int kLinesD = D / 32;          // 128-byte lines of a row of D floats
+                const int ld = lane < kLinesD ? lane : 0;
+                // W_o: up to three rows, one per helper wavefront
+                {
+                    const int row = other + G * hw;
+                    if (hw < (D + G - 1) / G && row < D) touched += w.wo[static_cast<size_t>(row) * D + ld * 32];
+                }
+                // FFN1: the head workgroup's eight items of two rows each, dealt to the five helpers
+                for (int wv = hw; wv < kPersistWaves; wv += kPersistWaves - (D + G - 1) / G) {
+                    const int item = other + G * wv;
+                    if (item < NIT) {
+                        touched += w.w1[static_cast<size_t>(2 * item) * D + ld * 32];
+                        touched += w.w1[static_cast<size_t>(2 * item + 1) * D + ld * 32];
+                    }
+                }
+                // FFN2: up to three rows of F floats
+                {
+                    const int row = other + G * hw;
+                    if (hw < (D + G - 1) / G && row < D) {
+#pragma unroll
+                        for (int part = 0; part < (F + 2047) / 2048; part++)
+                            touched += w.w2[static_cast<size_t>(row) * F + (part * 2048 + lane * 32) % F];
+                    }
+                }
+                asm volatile("" ::"v"(touched));
+            }
             if constexpr (F > 2048) {
                 if (early_ffn1 && wave < 2 * ((D + G - 1) / G)) {
                     const int w3 = wave - (D + G - 1) / G;  // the wavefront whose row this one touches
