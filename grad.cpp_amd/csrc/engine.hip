@@ -11,6 +11,7 @@
 #include "kernels_gemv.h"
 #include "kernels_persist.h"
 #include "kernels_pick.h"
+#include "kernels_xcd.h"
 
 #include <algorithm>
 #include <cmath>
@@ -142,8 +143,16 @@ struct Model {
     float *rope_cos = nullptr, *rope_sin = nullptr;  // (max_len, head_size/2)
     std::vector<Placement> place;                    // file order
 
+    // The XCD-sharded persistent kernel reads the weights from a second copy laid
+    // out as one contiguous stream per workgroup (kernels_xcd.h); built by the
+    // first session that uses it.
+    mutable std::mutex xcd_mutex;
+    mutable char* xcd_stream = nullptr;
+    mutable XcdGeom xcd_geom{};
+
     ~Model() {
         if (blob) (void)hipFree(blob);
+        if (xcd_stream) (void)hipFree(xcd_stream);
     }
 };
 
@@ -368,6 +377,15 @@ struct Session {
     unsigned long long* prof = nullptr;  // phase timestamps when GRADHIP_PROF_DUMP is set
     int prof_cap = 0;
     size_t persist_lds = 0;
+    // ... its XCD-sharded form (kernels_xcd.h)
+    bool xcd = false;
+    bool xcd_row_lds = false;
+    Cell* xcells = nullptr;
+    unsigned xcd_cells_count = 0;
+    unsigned xcd_launches = 0;
+    unsigned xcd_ring_units = 0, xcd_ring_units_wg0 = 0;
+    size_t xcd_lds = 0;
+    bool xcd_all_slices = false;  // every workgroup of an XCD takes a slice of the attention at any context
 
     float* host_logits = nullptr;  // pinned, B * V
     int* host_ids = nullptr;       // pinned staging for ids
@@ -408,7 +426,7 @@ struct Session {
                         static_cast<void*>(attn_part), static_cast<void*>(attn_tickets),
                         static_cast<void*>(tok), static_cast<void*>(hist), static_cast<void*>(st),
                         static_cast<void*>(uniforms),
-                        static_cast<void*>(logit_log), static_cast<void*>(cells),
+                        static_cast<void*>(logit_log), static_cast<void*>(cells), static_cast<void*>(xcells),
                         static_cast<void*>(ctl), static_cast<void*>(pp_x), static_cast<void*>(pp_q),
                         static_cast<void*>(pp_attn), static_cast<void*>(pp_norm),
                         static_cast<void*>(pp_hidden), static_cast<void*>(score_logits)})
@@ -688,6 +706,149 @@ static PersistKernel persist_kernel_for(const Shape& sh, bool row_lds, bool feed
     return row_lds ? persist_kernel_of<true, false>(sh) : persist_kernel_of<false, false>(sh);
 }
 
+
+// ---- the XCD-sharded form of the persistent kernel (kernels_xcd.h)
+
+using XcdKernel = void (*)(const XcdParams);
+
+static XcdKernel xcd_kernel_for(const Shape& sh, bool row_lds, bool feed) {
+    if (!sh.modern() || sh.head_size() != 64 || sh.d_model != 768) return nullptr;
+    if (feed) return row_lds ? xcd_decode_kernel<3, true, true> : xcd_decode_kernel<3, false, true>;
+    return row_lds ? xcd_decode_kernel<3, true, false> : xcd_decode_kernel<3, false, false>;
+}
+
+// Splits the model over eight XCDs: heads g and g + 8, and a run of hidden units
+// sized so that every XCD streams about the same number of bytes per layer.
+// False when the kernel's split does not fit the shape.
+static bool xcd_geometry(const Shape& sh, XcdGeom& gm) {
+    if (!xcd_kernel_for(sh, true, false)) return false;
+    const int D = sh.d_model, F = sh.d_ff(), H = sh.heads;
+    if (H < kXcds || H > 2 * kXcds || F % 4 != 0 || sh.layers < 1 || sh.max_len > 4096) return false;
+    gm = XcdGeom{};
+    gm.D = D;
+    gm.F = F;
+    gm.V = sh.vocab;
+    gm.L = sh.layers;
+    gm.H = H;
+    const double per_head = 4.0 * 64.0 * D, per_unit = 3.0 * D;
+    const double target = (H * per_head + F * per_unit) / kXcds;
+    double want_sum = 0.0;
+    int at = 0;
+    for (int g = 0; g < kXcds; g++) {
+        XcdShard& x = gm.shard[g];
+        x.nh = g + kXcds < H ? 2 : 1;
+        x.head[0] = g;
+        x.head[1] = g + kXcds < H ? g + kXcds : g;
+        want_sum += (target - x.nh * per_head) / per_unit;
+        int end = g == kXcds - 1 ? F : static_cast<int>(std::lround(want_sum / 4.0)) * 4;
+        end = std::min(std::max(end, at), F);
+        x.u0 = at;
+        x.nu = end - at;
+        at = end;
+        if (x.nu < kWgPerXcd || x.nu > 512) return false;  // every workgroup owns a unit; the XCD's units fit the LDS row
+    }
+    unsigned stride = 0;
+    for (int g = 0; g < kXcds; g++)
+        for (int r = 0; r < kWgPerXcd; r++) {
+            const XcdWg w = xcd_wg(gm, g, r);
+            if (w.nu < 1 || w.nu > kXcdMaxUnitsPerWg) return false;
+            stride = std::max(stride, w.layers_units + w.logits_units);
+        }
+    gm.stride_units = stride;
+    return true;
+}
+
+// One block of a weight matrix on its way into a workgroup's stream: rows x cols
+// floats from blob[src + row * src_ld] to stream[dst + row * dst_ld], each column
+// multiplied by a norm gain when gamma >= 0 (the gain of the norm in front of the
+// product is folded into the weights: (g * x) . w == x . (g * w)).
+struct XcdCopy {
+    unsigned long long dst, src;
+    long long gamma;
+    int rows, cols, src_ld, dst_ld;
+};
+
+__global__ void xcd_copy_kernel(const XcdCopy* list, const float* __restrict__ blob, float* __restrict__ out) {
+    const XcdCopy c = list[blockIdx.x];
+    const int n = c.rows * c.cols;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int row = i / c.cols, col = i - row * c.cols;
+        float v = blob[c.src + static_cast<size_t>(row) * c.src_ld + col];
+        if (c.gamma >= 0) v *= blob[c.gamma + col];
+        out[c.dst + static_cast<size_t>(row) * c.dst_ld + col] = v;
+    }
+}
+
+// Builds the per-workgroup weight streams of a model (once).
+static void xcd_build_stream(const Model& m) {
+    std::lock_guard<std::mutex> lock(m.xcd_mutex);
+    if (m.xcd_stream) return;
+    XcdGeom gm;
+    if (!xcd_geometry(m.shape, gm)) throw ApiError{GH_ERR_RUNTIME, "no XCD split for this model shape"};
+    const size_t D = gm.D, F = gm.F, RW = D / kWgPerXcd;
+    const size_t stride_floats = static_cast<size_t>(gm.stride_units) * kXcdUnit / 4;
+    auto at = [&](const float* ptr) { return static_cast<unsigned long long>(ptr - m.blob); };
+    std::vector<XcdCopy> list;
+    for (int g = 0; g < kXcds; g++)
+        for (int r = 0; r < kWgPerXcd; r++) {
+            const XcdWg w = xcd_wg(gm, g, r);
+            const XcdShard& sh = gm.shard[g];
+            const size_t base = static_cast<size_t>(g * kWgPerXcd + r) * stride_floats;
+            for (int l = 0; l < gm.L; l++) {
+                const LayerWeights& lw = m.layers[l];
+                const size_t lb = base + static_cast<size_t>(l) * (w.layer_bytes / 4);
+                // pairs of Q / K / V rows: pair i of the XCD is (head slot, section, j)
+                for (int q = 0; q < w.ppw; q++) {
+                    const int pi = r * w.ppw + q, hi = pi / 96, rem = pi % 96, sec = rem / 32, j = rem % 32;
+                    const size_t row = static_cast<size_t>(sec) * D + static_cast<size_t>(sh.head[hi]) * 64 + 2 * j;
+                    const size_t pb = lb + static_cast<size_t>(q) * (w.pair_bytes / 4);
+                    list.push_back({pb, at(lw.wqkv) + row * D, static_cast<long long>(at(lw.g1)), 2,
+                                    static_cast<int>(D), static_cast<int>(D), static_cast<int>(D)});
+                    list.push_back({pb + 2 * D, at(lw.bqkv) + row, -1, 1, 2, 2, 2});
+                }
+                // W_o: this workgroup's rows, the columns of the XCD's heads
+                for (int hi = 0; hi < w.nh; hi++)
+                    list.push_back({lb + w.o_wo / 4 + static_cast<size_t>(hi) * 64,
+                                    at(lw.wo) + (static_cast<size_t>(r) * RW) * D + static_cast<size_t>(sh.head[hi]) * 64,
+                                    -1, static_cast<int>(RW), 64, static_cast<int>(D), w.KC});
+                list.push_back({lb + w.o_bo / 4, at(lw.bo) + static_cast<size_t>(r) * RW, -1, 1, static_cast<int>(RW),
+                                static_cast<int>(RW), static_cast<int>(RW)});
+                // gate and up rows of this workgroup's hidden units (row 2u gate, 2u + 1 up)
+                list.push_back({lb + w.o_gu / 4, at(lw.w1) + static_cast<size_t>(2 * w.ub) * D,
+                                static_cast<long long>(at(lw.g2)), 2 * w.nu, static_cast<int>(D),
+                                static_cast<int>(D), static_cast<int>(D)});
+                // W_down: this workgroup's rows, the columns of the XCD's hidden units
+                list.push_back({lb + w.o_dn / 4, at(lw.w2) + (static_cast<size_t>(r) * RW) * F + static_cast<size_t>(w.u0),
+                                -1, static_cast<int>(RW), w.UG, static_cast<int>(F), w.UG});
+            }
+            // its rows of the logits matrix, with the final norm's gain
+            if (w.nrows > 0)
+                list.push_back({base + static_cast<size_t>(w.layers_units) * kXcdUnit / 4,
+                                at(m.E) + static_cast<size_t>(w.v0) * D, static_cast<long long>(at(m.gf)), w.nrows,
+                                static_cast<int>(D), static_cast<int>(D), static_cast<int>(D)});
+        }
+    const size_t total = static_cast<size_t>(kXcds * kWgPerXcd) * stride_floats;
+    char* stream = nullptr;
+    XcdCopy* dlist = nullptr;
+    HIP_CHECK(hipMalloc(&stream, total * sizeof(float)));
+    try {
+        HIP_CHECK(hipMemset(stream, 0, total * sizeof(float)));
+        HIP_CHECK(hipMalloc(&dlist, list.size() * sizeof(XcdCopy)));
+        HIP_CHECK(hipMemcpy(dlist, list.data(), list.size() * sizeof(XcdCopy), hipMemcpyHostToDevice));
+        hipLaunchKernelGGL(xcd_copy_kernel, dim3(static_cast<unsigned>(list.size())), dim3(256), 0, nullptr, dlist,
+                           m.blob, reinterpret_cast<float*>(stream));
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipDeviceSynchronize());
+    } catch (...) {
+        if (dlist) (void)hipFree(dlist);
+        (void)hipFree(stream);
+        throw;
+    }
+    HIP_CHECK(hipFree(dlist));
+    m.xcd_geom = gm;
+    m.xcd_stream = stream;
+}
+
 static const char* persist_unavailable(const Session& s, int lds_bytes, int cus) {
     const Shape& sh = s.m->shape;
     if (s.B != 1) return "the persistent engine decodes one sequence";
@@ -736,6 +897,7 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
         const unsigned long long last = (static_cast<unsigned long long>(s.epoch) + n_steps + 2ull) * per_step + 8ull;
         if (last >= 0xF0000000ull) {
             HIP_CHECK(hipMemsetAsync(s.cells, 0, s.cells_count * sizeof(Cell), s.stream));
+            if (s.xcells) HIP_CHECK(hipMemsetAsync(s.xcells, 0, s.xcd_cells_count * sizeof(Cell), s.stream));
             s.epoch = 1;
         }
     }
@@ -799,8 +961,25 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     k.work_stride = s.work_stride;
     k.sort_cap = kPickWorkFloats;
 
-    PersistKernel kernel = persist_kernel_for(sh, s.pick_row_in_lds, feed);
-    hipLaunchKernelGGL(kernel, dim3(s.persist_grid), dim3(kPersistThreads), s.persist_lds, s.stream, p);
+    if (s.xcd) {
+        XcdParams x{};
+        x.b = p;
+        x.gm = m.xcd_geom;
+        x.stream = m.xcd_stream;
+        x.xc = s.xcells;
+        x.ring_units = s.xcd_ring_units;
+        x.ring_units_wg0 = s.xcd_ring_units_wg0;
+        x.launch_base = s.xcd_launches * kWgPerXcd;
+        // Eight slices per head keep the merge short; contexts beyond 256 positions give
+        // every workgroup of the XCD a slice.
+        x.attn_slices = (s.xcd_all_slices || s.pos + n_steps > 256) ? 0 : 8;
+        s.xcd_launches++;
+        hipLaunchKernelGGL(xcd_kernel_for(sh, s.xcd_row_lds, feed), dim3(kXcds * kWgPerXcd), dim3(kXcdThreads),
+                           s.xcd_lds, s.stream, x);
+    } else {
+        PersistKernel kernel = persist_kernel_for(sh, s.pick_row_in_lds, feed);
+        hipLaunchKernelGGL(kernel, dim3(s.persist_grid), dim3(kPersistThreads), s.persist_lds, s.stream, p);
+    }
     HIP_CHECK(hipGetLastError());
 
     // Host mirrors.  Logits are produced by the last prompt step and every later one.
@@ -1006,6 +1185,46 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
                     reinterpret_cast<const void*>(persist_kernel_for(sh, s.pick_row_in_lds, feed)),
                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(s.persist_lds)));
             s.launches_per_step = 1;
+
+            // The XCD-sharded form, where the chip and the shape allow it: 8 XCDs of 32
+            // compute units, and a ring of a power-of-two size beside the work area
+            // (workgroup 0's ring is smaller when the pick keeps its row in LDS).
+            XcdGeom gm;
+            if ((o.flags & GH_FLAG_CLASSIC_PERSISTENT) == 0 && prop.multiProcessorCount == kXcds * kWgPerXcd
+                && xcd_geometry(sh, gm) && s.pages_per_seq <= 1024) {
+                const size_t statics = 4096;  // the kernel's static LDS (control words, the pick's scratch), rounded up
+                const size_t work = (2 * d + kWgPerXcd * kApCells + 512 + kXcdRowWaves * 128 + 192 + s.pages_per_seq)
+                                    * sizeof(float);
+                const size_t pick_small = kPickWorkFloats * sizeof(float);
+                const size_t pick_row = (V + kPickWorkFloats) * sizeof(float);
+                size_t ring = 128 * 1024;
+                while (ring + std::max(work, pick_small) + statics > static_cast<size_t>(lds_bytes)) ring /= 2;
+                size_t ring0 = ring;
+                s.xcd_row_lds = false;
+                if (!s.pick_global_scratch) {
+                    size_t rr = ring;
+                    while (rr >= 32 * 1024 && rr + std::max(work, pick_row) + statics > static_cast<size_t>(lds_bytes)) rr /= 2;
+                    if (rr >= 32 * 1024) {
+                        ring0 = rr;
+                        s.xcd_row_lds = true;
+                    }
+                }
+                if (ring >= 64 * 1024) {
+                    xcd_build_stream(m);
+                    s.xcd = true;
+                    s.xcd_all_slices = (o.flags & GH_FLAG_SMALL_ATTENTION_CHUNKS) != 0;
+                    s.xcd_ring_units = static_cast<unsigned>(ring / kXcdUnit);
+                    s.xcd_ring_units_wg0 = static_cast<unsigned>(ring0 / kXcdUnit);
+                    s.xcd_lds = std::max(ring + work, ring0 + std::max(work, s.xcd_row_lds ? pick_row : pick_small));
+                    const XcdCells cl = xcd_cells(m.xcd_geom);
+                    s.xcd_cells_count = cl.total;
+                    dev_alloc(s.xcells, cl.total);
+                    for (const bool feed : {false, true})
+                        HIP_CHECK(hipFuncSetAttribute(
+                            reinterpret_cast<const void*>(xcd_kernel_for(sh, s.xcd_row_lds, feed)),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(s.xcd_lds)));
+                }
+            }
         }
     }
 

@@ -73,6 +73,7 @@ struct PersistCtl {
     unsigned where;     // phase tag it was waiting for (diagnostics)
     unsigned pad[30];
     unsigned arrive[16 * 32];  // logits-complete counters, one per 128-byte line
+    unsigned xcd_count[8 * 32];  // workgroups that have started on each XCD, one counter per line (kernels_xcd.h)
 };
 
 struct PersistParams {
@@ -198,9 +199,12 @@ __device__ __forceinline__ void feed_put(const PersistParams& p, int i_pick, int
 // workgroup's logits rows have landed, picks, records the token in the history
 // and publishes it in the token cell.  The other workgroups return at once and
 // learn the token from the cell.  False: the wait was abandoned.
-template <bool ROW_LDS, bool FEED>
+// NT: threads of the workgroup (all of them call).  tok_cell: where the token is
+// published.  chosen_out: the pick, for every thread of workgroup 0.
+template <bool ROW_LDS, bool FEED, int NT = kPersistThreads>
 __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds, int i_pick,
-                                    unsigned arrive_gen, unsigned tok_tag, bool wait_logits, int grid) {
+                                    unsigned arrive_gen, unsigned tok_tag, bool wait_logits, int grid,
+                                    Cell* tok_cell, int* chosen_out = nullptr) {
     if (blockIdx.x != 0) return true;
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));  // nothing of the pick is computed ahead of the token loop
@@ -216,7 +220,7 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
         const unsigned stop = __hip_atomic_load(p.stop_request, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         if (__builtin_amdgcn_readfirstlane(stop) != 0u) {
             if (tid == 0) {
-                cell_put((p.cells + 6 * p.d + p.F), __int_as_float(-1), tok_tag);
+                cell_put(tok_cell, __int_as_float(-1), tok_tag);
                 feed_put(p, i_pick, -1);
             }
             return false;
@@ -255,11 +259,12 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
     }
     unsigned long long* pp = (p.prof && i_pick < 1024) ? p.prof + p.prof_cap / 2 + 4 * i_pick : nullptr;
     if (pp && tid == 0) pp[0] = __builtin_amdgcn_s_memrealtime();
-    const int chosen = ROW_LDS ? pick_body<true, kPersistThreads>(pk, 0, lds, lds + pk.V, u)
-                               : pick_body<true, kPersistThreads>(pk, 0, pk.work, lds, u);
+    const int chosen = ROW_LDS ? pick_body<true, NT>(pk, 0, lds, lds + pk.V, u)
+                               : pick_body<true, NT>(pk, 0, pk.work, lds, u);
+    if (chosen_out) *chosen_out = chosen;
     if (tid == 0) {
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        cell_put((p.cells + 6 * p.d + p.F), __int_as_float(chosen), tok_tag);
+        cell_put(tok_cell, __int_as_float(chosen), tok_tag);
         if constexpr (FEED) feed_put(p, i_pick, chosen);
         if (pp) pp[1] = __builtin_amdgcn_s_memrealtime();
     }
@@ -423,7 +428,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         if ((!FEED || !ended) && i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick)) {
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
-            if (!persist_pick<ROW_LDS, FEED>(p, lds, i_pick, arrive_gen, tt, s > 0, G)) return;
+            if (!persist_pick<ROW_LDS, FEED>(p, lds, i_pick, arrive_gen, tt, s > 0, G, p.cells + 6 * p.d + p.F)) return;
             i_pick++;
             if (wg == 0) {
                 // the pick used the whole LDS; restore the page table

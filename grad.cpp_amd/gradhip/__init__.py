@@ -21,6 +21,7 @@ ENGINE_AUTO, ENGINE_GRAPH, ENGINE_EAGER, ENGINE_PERSISTENT = range(4)
 FLAG_PICK_GLOBAL_SCRATCH = 1
 FLAG_STEPWISE_PROMPT = 2
 FLAG_SMALL_ATTENTION_CHUNKS = 4
+FLAG_CLASSIC_PERSISTENT = 8
 
 
 class DeviceError(RuntimeError):

@@ -120,6 +120,11 @@ enum { GH_FLAG_STEPWISE_PROMPT = 2 };
  * contexts. */
 enum { GH_FLAG_SMALL_ATTENTION_CHUNKS = 4 };
 
+/* Keep the persistent engine on its all-to-all kernel (every phase exchanged among
+ * all 256 workgroups) where the XCD-sharded kernel would otherwise run; for
+ * comparing the two and for testing the one that is not the default. */
+enum { GH_FLAG_CLASSIC_PERSISTENT = 8 };
+
 /* InferenceSession::InferenceSession (inference.cpp:121-148): allocates the
  * paged KV cache (2 * layers * max_len * d_model floats per sequence) and the
  * per-step scratch, and records the step graph. */
