@@ -378,7 +378,8 @@ struct Session {
     int prof_cap = 0;
     size_t persist_lds = 0;
     // ... its XCD-sharded form (kernels_xcd.h)
-    bool xcd = false;
+    bool xcd = false;         // the kernel and its buffers are ready
+    bool xcd_always = false;  // GH_FLAG_XCD_PERSISTENT: every launch takes it
     bool xcd_row_lds = false;
     Cell* xcells = nullptr;
     unsigned xcd_cells_count = 0;
@@ -408,8 +409,10 @@ struct Session {
                 if (std::FILE* f = std::fopen(std::getenv("GRADHIP_PROF_DUMP"), "w")) {
                     for (size_t i = 0; i < host.size() / 2 && host[i]; i++) std::fprintf(f, "%llu\n", host[i]);
                     std::fprintf(f, "0\n");
-                    for (size_t i = host.size() / 2; i + 3 < host.size() && host[i]; i += 4)
+                    for (size_t i = host.size() / 2; i + 3 < host.size() - 112 && host[i]; i += 4)
                         std::fprintf(f, "%llu\n%llu\n%llu\n", host[i + 2], host[i], host[i + 1]);
+                    std::fprintf(f, "0\n");
+                    for (size_t i = host.size() - 112; i < host.size(); i++) std::fprintf(f, "%llu\n", host[i]);
                     std::fclose(f);
                 }
             }
@@ -709,6 +712,9 @@ static PersistKernel persist_kernel_for(const Shape& sh, bool row_lds, bool feed
 
 // ---- the XCD-sharded form of the persistent kernel (kernels_xcd.h)
 
+// First position of a launch from which the XCD-sharded kernel is the default.
+constexpr int kXcdFromPosition = 1536;
+
 using XcdKernel = void (*)(const XcdParams);
 
 static XcdKernel xcd_kernel_for(const Shape& sh, bool row_lds, bool feed) {
@@ -961,7 +967,9 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     k.work_stride = s.work_stride;
     k.sort_cap = kPickWorkFloats;
 
-    if (s.xcd) {
+    // The XCD-sharded kernel wins where attention is long (it spreads a head's context over
+    // the workgroups of an XCD): launches that start deep in the context take it.
+    if (s.xcd && (s.xcd_always || s.pos >= kXcdFromPosition)) {
         XcdParams x{};
         x.b = p;
         x.gm = m.xcd_geom;
@@ -1190,10 +1198,14 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
             // compute units, and a ring of a power-of-two size beside the work area
             // (workgroup 0's ring is smaller when the pick keeps its row in LDS).
             XcdGeom gm;
-            if ((o.flags & GH_FLAG_CLASSIC_PERSISTENT) == 0 && prop.multiProcessorCount == kXcds * kWgPerXcd
-                && xcd_geometry(sh, gm) && s.pages_per_seq <= 1024) {
+            const bool xcd_wanted = (o.flags & GH_FLAG_XCD_PERSISTENT) != 0
+                                    || ((o.flags & GH_FLAG_CLASSIC_PERSISTENT) == 0 && sh.max_len > kXcdFromPosition);
+            if ((o.flags & GH_FLAG_XCD_PERSISTENT) != 0 && (o.flags & GH_FLAG_CLASSIC_PERSISTENT) != 0)
+                throw ApiError{GH_ERR_INVALID_ARGUMENT, "GH_FLAG_CLASSIC_PERSISTENT and GH_FLAG_XCD_PERSISTENT exclude each other"};
+            if (xcd_wanted && prop.multiProcessorCount == kXcds * kWgPerXcd && xcd_geometry(sh, gm)
+                && s.pages_per_seq <= 1024) {
                 const size_t statics = 4096;  // the kernel's static LDS (control words, the pick's scratch), rounded up
-                const size_t work = (2 * d + kWgPerXcd * kApCells + 512 + kXcdRowWaves * 128 + 192 + s.pages_per_seq)
+                const size_t work = (2 * d + kWgPerXcd * kApCells + 512 + kXcdRowWaves * (128 + 32) + 192 + s.pages_per_seq)
                                     * sizeof(float);
                 const size_t pick_small = kPickWorkFloats * sizeof(float);
                 const size_t pick_row = (V + kPickWorkFloats) * sizeof(float);
@@ -1212,6 +1224,7 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
                 if (ring >= 64 * 1024) {
                     xcd_build_stream(m);
                     s.xcd = true;
+                    s.xcd_always = (o.flags & GH_FLAG_XCD_PERSISTENT) != 0;
                     s.xcd_all_slices = (o.flags & GH_FLAG_SMALL_ATTENTION_CHUNKS) != 0;
                     s.xcd_ring_units = static_cast<unsigned>(ring / kXcdUnit);
                     s.xcd_ring_units_wg0 = static_cast<unsigned>(ring0 / kXcdUnit);

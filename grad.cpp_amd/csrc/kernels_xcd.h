@@ -56,7 +56,7 @@ constexpr int kXcdRelayWave = 6;      // sums the partials of this workgroup's r
 constexpr int kXcdAttnWave = 7;       // attention of one slice (P2); takes no part in anything else
 constexpr int kXcds = 8, kWgPerXcd = 32;
 constexpr int kXcdUnit = 1024;        // bytes one streamer instruction moves
-constexpr int kXcdDepth = 12;         // loads a streamer keeps in flight
+constexpr int kXcdDepth = 4;          // loads a streamer keeps in flight
 constexpr int kAuxNonTemporal = 2;    // nt on gfx94x / gfx950 buffer instructions
 constexpr int kApCells = 66;          // cells of one attention partial: acc[64], m, l
 constexpr int kXcdMaxUnitsPerWg = 2 * kXcdTeamWaves;
@@ -196,7 +196,14 @@ __device__ __forceinline__ void wave_sum2(float& a, float& b) {
     b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(b), 63));
 }
 
-// A cell written for readers inside the XCD: an ordinary store, which lands in the L2.
+// A cell written for readers inside the XCD.  Also a device-scope (write-through)
+// store: an ordinary store may sit in the compute unit's write path for
+// microseconds while the memory system is busy (a two-workgroup ping-pong under a
+// streaming load: 0.25 us per hand-off with write-through stores, 8 us with
+// ordinary ones), and every workgroup of the XCD is waiting for this one.
+#ifndef GH_XCD_BAR_SLEEP
+#define GH_XCD_BAR_SLEEP 1
+#endif
 __device__ __forceinline__ void cell_put_local(Cell* c, float v, unsigned tag) {
     v2i w;
     w.x = __float_as_int(v);
@@ -228,10 +235,18 @@ __device__ __forceinline__ void xcd_give_up(const XcdWait& w, unsigned where) {
 // cells other XCDs wrote, non-temporal for cells of this XCD.  False: abandoned.
 template <int AUX>
 __device__ __forceinline__ bool xcd_gather(const Cell* src, int n, unsigned tag, float* dst, int ctid,
-                                           const XcdWait& w) {
+                                           const XcdWait& w, unsigned* rounds = nullptr, unsigned* first_trip = nullptr) {
     const __amdgpu_buffer_rsrc_t rs = make_buffer(src, static_cast<unsigned>(n) * 8u);
     const int itag = static_cast<int>(tag);
     unsigned spins = 0;
+    if (first_trip) {
+        // diagnostics: one poll, timed from issue to return
+        const unsigned t0 = static_cast<unsigned>(__builtin_amdgcn_s_memtime());
+        const v4i c = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<unsigned>(2 * ctid < n ? 2 * ctid : 0) * 8u, 0, AUX);
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(c) : "memory");
+        *first_trip += static_cast<unsigned>(__builtin_amdgcn_s_memtime()) - t0;
+    }
+#pragma nounroll
     for (;;) {
         bool ok = true;
         for (int i = 2 * ctid; i < n; i += 2 * kXcdTeamLanes) {
@@ -240,7 +255,10 @@ __device__ __forceinline__ bool xcd_gather(const Cell* src, int n, unsigned tag,
             dst[i] = __int_as_float(c.x);
             if (i + 1 < n) dst[i + 1] = __int_as_float(c.z);
         }
-        if (ok) return true;
+        if (ok) {
+            if (rounds) *rounds += spins;
+            return true;
+        }
         ++spins;
         if (spins > w.spin_limit || w.ctl[kXAbandon] != 0u
             || ((spins & 63u) == 0u
@@ -255,27 +273,38 @@ __device__ __forceinline__ bool xcd_gather(const Cell* src, int n, unsigned tag,
 // visible to all of them after it.  (The hardware barrier would include the
 // streamers, which must never wait for anybody.)  gen counts this wavefront's
 // barriers.  False: abandoned.
-__device__ __forceinline__ bool xcd_team_sync(const XcdWait& w, unsigned& gen, int lane) {
+__device__ __forceinline__ bool xcd_team_sync(const XcdWait& w, unsigned& gen, int lane, unsigned* rounds = nullptr) {
     gen += kXcdTeamWaves;
     lds_settle();
     if (lane == 0)
         __hip_atomic_fetch_add((__attribute__((address_space(3))) unsigned*)(&w.ctl[kXBar]), 1u, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_WORKGROUP);
     unsigned spins = 0;
+    // A waiting wavefront sleeps between looks: seven wavefronts reading the counter
+    // as fast as they can take the LDS and the issue slots from the ones that work
+    // (the attention wavefront ran four times slower beside such a loop).
+#pragma nounroll
     while (static_cast<int>(w.ctl[kXBar] - gen) < 0) {
-        if (w.ctl[kXAbandon] != 0u) return false;
-        if (++spins > (1u << 24)) {
-            xcd_give_up(w, 0xFFFFFFF0u);
-            return false;
+        ++spins;
+        if ((spins & 15u) == 0u) {
+            if (w.ctl[kXAbandon] != 0u) return false;
+            if (spins > (1u << 22)) {
+                xcd_give_up(w, 0xFFFFFFF0u);
+                return false;
+            }
         }
+        __builtin_amdgcn_s_sleep(GH_XCD_BAR_SLEEP);
     }
+    asm volatile("" ::: "memory");
+    if (rounds) *rounds += spins;
     return true;
 }
 
 // Waits until the streamers have written every unit below `units` (counted from the
 // start of the launch) into the ring.
-__device__ __forceinline__ bool xcd_wait_filled(const XcdWait& w, unsigned units) {
+__device__ __forceinline__ bool xcd_wait_filled(const XcdWait& w, unsigned units, unsigned* stalled = nullptr) {
     unsigned spins = 0;
+#pragma nounroll
     for (;;) {
         bool ok = true;
 #pragma unroll
@@ -286,13 +315,15 @@ __device__ __forceinline__ bool xcd_wait_filled(const XcdWait& w, unsigned units
         }
         if (ok) {
             asm volatile("" ::: "memory");  // ring reads stay behind the wait
+            if (stalled) *stalled += spins;
             return true;
         }
         if (w.ctl[kXAbandon] != 0u) return false;
-        if (++spins > (1u << 24)) {
+        if (++spins > (1u << 22)) {
             xcd_give_up(w, 0xFFFFFFF1u);
             return false;
         }
+        __builtin_amdgcn_s_sleep(1);
     }
 }
 
@@ -317,84 +348,103 @@ __device__ __forceinline__ bool xcd_wants_logits(const PersistParams& p, int s) 
 // ring, kXcdDepth loads in flight, never writing a unit before every compute
 // wavefront is past the unit it overwrites.  unit_base: units of the launch before
 // step s0 (updated); count: units this wavefront has written (updated).
+//
+// Steps without logits (all but the last of a prompt run) come first in a launch
+// and are shorter; both kinds start at the beginning of the workgroup's stream.
+// The loop is straight-line code over compile-time register indices: a data-
+// dependent exit from it would turn the registers in flight into an array in
+// scratch memory, with a wait behind every load.
+struct XcdCursor {
+    unsigned j;      // this wavefront's unit number inside the step (unit 4 j + sw of the step)
+    unsigned per;    // units of this wavefront in the current step
+    unsigned shorts; // steps without logits still to come, the current one included
+    unsigned gbase;  // units of the launch before the current step
+};
+
+__device__ __forceinline__ void xcd_cursor_next(XcdCursor& c, unsigned per_short, unsigned per_full) {
+    c.j++;
+    const bool wrap = c.j == c.per;
+    c.gbase += wrap ? 4u * c.per : 0u;
+    c.j = wrap ? 0u : c.j;
+    const unsigned left = (wrap && c.shorts > 0u) ? c.shorts - 1u : c.shorts;
+    c.per = (wrap && left == 0u) ? per_full : c.per;
+    c.shorts = left;
+}
+
 __device__ inline void xcd_stream(const XcdParams& p, const XcdWg& me, const char* src, char* ring,
                                   unsigned ring_units, const XcdWait& w, int sw, int lane, int s0, int s1,
                                   unsigned& unit_base, unsigned& count) {
-    const unsigned mask = ring_units * kXcdUnit - 1u;
-    auto units_of = [&](int s) { return me.layers_units + (xcd_wants_logits(p.b, s) ? me.logits_units : 0u); };
     if (s0 >= s1) return;
-    // issue side
-    int is = s0;
-    unsigned iu = static_cast<unsigned>(sw), in = units_of(s0);
-    // write side
-    int ws = s0;
-    unsigned wu = static_cast<unsigned>(sw), wn = in, wbase = unit_base;
+    const unsigned mask = ring_units * kXcdUnit - 1u;
+    const unsigned per_short = me.layers_units / kXcdStreamWaves;
+    const unsigned per_full = (me.layers_units + me.logits_units) / kXcdStreamWaves;
+    // steps [0, n_short) of the launch go without logits
+    const int n_short = p.b.logit_log ? 0 : max(0, min(p.b.n_prompt - 1, p.b.n_steps - 1));
+    const unsigned shorts = static_cast<unsigned>(max(0, min(s1, n_short) - s0));
+    const unsigned fulls = static_cast<unsigned>(s1 - s0) - shorts;
+    unsigned total = shorts * per_short + fulls * per_full;  // units of this wavefront
+    XcdCursor ci{0u, shorts > 0u ? per_short : per_full, shorts, unit_base};
+    XcdCursor cw = ci;
+    unsigned issued = 0;
     unsigned space_end = 0;  // units below this may be written
-    const char* lane_src = src + lane * 16;
+    const char* lane_src = src + lane * 16 + sw * kXcdUnit;
     auto issue = [&](v4f& dst) {
-        while (is < s1 && iu >= in) {
-            is++;
-            iu = static_cast<unsigned>(sw);
-            if (is < s1) in = units_of(is);
-        }
         // past the end: a harmless reload of the first unit, so that no load sits under a branch
-        const unsigned at = is < s1 ? iu : static_cast<unsigned>(sw);
-        dst = *reinterpret_cast<const v4f*>(lane_src + static_cast<size_t>(at) * kXcdUnit);
-        iu += kXcdStreamWaves;
+        const unsigned at = issued < total ? ci.j : 0u;
+        dst = *reinterpret_cast<const v4f*>(lane_src + static_cast<size_t>(at) * (kXcdStreamWaves * kXcdUnit));
+        asm volatile("" ::: "memory");  // loads go out in this order: the oldest is the one written next
+        issued++;
+        xcd_cursor_next(ci, per_short, per_full);
     };
     v4f buf[kXcdDepth];
 #pragma unroll
     for (int i = 0; i < kXcdDepth; i++) issue(buf[i]);
-    bool live = true;
-    while (live) {
+    for (unsigned k0 = 0; k0 < total; k0 += kXcdDepth) {
 #pragma unroll
         for (int i = 0; i < kXcdDepth; i++) {
-            while (ws < s1 && wu >= wn) {
-                wbase += wn;
-                ws++;
-                wu = static_cast<unsigned>(sw);
-                if (ws < s1) wn = units_of(ws);
-            }
-            if (ws >= s1) {
-                live = false;
-                break;
-            }
-            const unsigned unit = wbase + wu;
-            if (static_cast<int>(unit - space_end) >= 0) {
-                unsigned spins = 0;
-                for (;;) {
-                    unsigned low = w.ctl[kXConsumed];
+            if (k0 + i < total) {
+                const unsigned unit = cw.gbase + 4u * cw.j + static_cast<unsigned>(sw);
+                if (static_cast<int>(unit - space_end) >= 0) {
+                    unsigned spins = 0;
+#pragma nounroll
+                    for (;;) {
+                        unsigned low = w.ctl[kXConsumed];
 #pragma unroll
-                    for (int q = 1; q < kXcdComputeWaves; q++) {
-                        const unsigned c = w.ctl[kXConsumed + q];
-                        low = c < low ? c : low;
+                        for (int q = 1; q < kXcdComputeWaves; q++) {
+                            const unsigned c = w.ctl[kXConsumed + q];
+                            low = c < low ? c : low;
+                        }
+                        space_end = low + ring_units;
+                        if (static_cast<int>(unit - space_end) < 0) break;
+                        if (w.ctl[kXDone] != 0u || w.ctl[kXAbandon] != 0u) {
+                            total = 0;  // leave: nothing more is written
+                            break;
+                        }
+                        if (++spins > (1u << 22)) {
+                            xcd_give_up(w, 0xFFFFFFF2u);
+                            total = 0;
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(2);
                     }
-                    space_end = low + ring_units;
-                    if (static_cast<int>(unit - space_end) < 0) break;
-                    if (w.ctl[kXDone] != 0u || w.ctl[kXAbandon] != 0u) {
-                        live = false;
-                        break;
-                    }
-                    if (++spins > (1u << 24)) {
-                        xcd_give_up(w, 0xFFFFFFF2u);
-                        live = false;
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(1);
                 }
-                if (!live) break;
+                if (total != 0u) {
+                    *reinterpret_cast<v4f*>(ring + ((unit * kXcdUnit + lane * 16) & mask)) = buf[i];
+                    count++;
+                    asm volatile("" ::: "memory");  // the unit, then its count: LDS keeps a wavefront's order
+                    if (lane == 0) w.ctl[kXFilled + sw] = count;
+                    xcd_cursor_next(cw, per_short, per_full);
+                }
             }
-            *reinterpret_cast<v4f*>(ring + ((unit * kXcdUnit + lane * 16) & mask)) = buf[i];
-            count++;
-            asm volatile("" ::: "memory");  // the unit, then its count: LDS keeps a wavefront's order
-            if (lane == 0) w.ctl[kXFilled + sw] = count;
-            wu += kXcdStreamWaves;
             issue(buf[i]);
+#ifdef GH_XCD_PACE
+            __builtin_amdgcn_s_sleep(GH_XCD_PACE);
+#endif
         }
     }
     // what is still in flight lands in registers only; let it arrive before leaving
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    unit_base = wbase;
+    unit_base = cw.gbase;
 }
 
 // KD = d_model / 256; head size 64.  FEED: the streaming variant.
@@ -434,8 +484,8 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
     float* xs1 = xs + D;                             // [D] after the attention half
     float* apbuf = xs1 + D;                          // [32 * kApCells] the XCD's attention partials
     float* hbuf = apbuf + kWgPerXcd * kApCells;      // [<= 512] the XCD's hidden units
-    float* att = hbuf + 512;                         // [row wavefronts][128] merged attention output
-    float* qkv7 = att + kXcdRowWaves * 128;          // [192] q, new key, new value (attention wavefront)
+    float* att = hbuf + 512;                         // [row wavefronts][128 + 32] merged attention output, merge factors
+    float* qkv7 = att + kXcdRowWaves * (128 + 32);   // [192] q, new key, new value (attention wavefront)
     int* ptab = reinterpret_cast<int*>(qkv7 + 192);  // [pages_per_seq]
     for (int i = tid; i < pb.kv.pages_per_seq; i += kXcdThreads) ptab[i] = pb.kv.page_table[i];
     __syncthreads();
@@ -463,12 +513,32 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
 
     const bool streamer = wave >= kXcdComputeWaves;
     const int sw = wave - kXcdComputeWaves;
+    // the wavefronts every workgroup of the XCD waits for go first when two are ready
+    if (wave == kXcdAttnWave || wave == kXcdRelayWave) __builtin_amdgcn_s_setprio(3);
+    else if (!streamer) __builtin_amdgcn_s_setprio(1);
     unsigned s_unit_base = 0, s_count = 0;  // streamer state
     unsigned unit_base = 0;                 // compute wavefronts: units of the launch before this step
     unsigned bar_gen = 0;
     int i_pick = 0;
     unsigned arrive_gen = pb.arrive_base;
     bool ended = false;
+    unsigned stall[13] = {};
+#ifdef GH_XCD_TICKS
+    unsigned dur[16] = {};
+    unsigned last_tick = 0;
+#define XTICK(k)                                                                  \
+    do {                                                                          \
+        const unsigned now_ = static_cast<unsigned>(__builtin_amdgcn_s_memtime()); \
+        dur[k] += now_ - last_tick;                                               \
+        last_tick = now_;                                                         \
+    } while (0)
+#define XTRIP(k) (&dur[k])
+#define XROUNDS(k, n) dur[k] += (n)
+#else
+#define XROUNDS(k, n) do { } while (0)
+#define XTICK(k) do { } while (0)
+#define XTRIP(k) nullptr
+#endif  // polls spent waiting for the ring, by phase (diagnostics)
     int n_stamp = 0;
     auto stamp = [&]() {
         if (pb.prof && wg == 0 && tid == 0 && n_stamp < pb.prof_cap / 2) pb.prof[n_stamp] = __builtin_amdgcn_s_memrealtime();
@@ -534,6 +604,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
             unsigned spins = 0;
             float tv = 0.0f;
+#pragma nounroll
             while (!cell_get(tok_cell, tt, tv)) {
                 if (++spins > pb.spin_limit || ctl[kXAbandon] != 0u
                     || ((spins & 63u) == 0u
@@ -552,6 +623,9 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
             }
         }
 
+#ifdef GH_XCD_TICKS
+        last_tick = static_cast<unsigned>(__builtin_amdgcn_s_memtime());
+#endif
         if (wave == kXcdAttnWave) {
             // ================= attention wavefront: P2 of every layer
             if (attn_wg) {
@@ -577,6 +651,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 };
                 fetch(0, 0);
                 for (int l = 0; l < L; l++) {
+                    XTICK(5);
                     // q (and the new key and value, if this slice holds the current position)
                     {
                         const unsigned t = tag_of(l, 0);
@@ -584,6 +659,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                         const int ncell = has_cur ? 192 : 64;
                         const __amdgpu_buffer_rsrc_t rs = make_buffer(src, static_cast<unsigned>(ncell) * 8u);
                         unsigned spins = 0;
+#pragma nounroll
                         for (;;) {
                             bool ok = true;
                             for (int i = 2 * lane; i < ncell; i += 128) {
@@ -602,7 +678,9 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                             }
                         }
                         lds_settle();
+                        XROUNDS(6, spins);
                     }
+                    XTICK(4);  // attention wavefront: 4 = wait for q, 5 = everything else
                     const float4 q4 = reinterpret_cast<const float4*>(qkv7)[dl];
                     float m = -INFINITY, lsum = 0.0f;
                     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -704,6 +782,9 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
         for (int j = ctid; j < D; j += kXcdTeamLanes) xs[j] = pb.E[static_cast<size_t>(tok) * D + j];
         if (!xcd_team_sync(wt, bar_gen, lane)) return;
 
+#ifdef GH_XCD_TICKS
+        last_tick = static_cast<unsigned>(__builtin_amdgcn_s_memtime());
+#endif
         for (int l = 0; l < L; l++) {
             const unsigned lay = static_cast<unsigned>(l) * me.layer_bytes;  // this layer in the step's stream
             auto unit_of = [&](unsigned off) { return unit_base + (off >> 10); };       // the unit holding byte off
@@ -721,7 +802,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 if (wave < me.ppw) {
                     const unsigned o = lay + static_cast<unsigned>(wave) * me.pair_bytes;
                     xcd_set_consumed(wt, wave, lane, unit_of(o));
-                    if (!xcd_wait_filled(wt, units_to(o + me.pair_bytes))) return;
+                    if (!xcd_wait_filled(wt, units_to(o + me.pair_bytes), &stall[0])) return;
                     const float rn = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(D) + kNormEps);
                     float a = 0.0f, c = 0.0f;
                     const unsigned base = unit_base * kXcdUnit + o + lane * 16;
@@ -745,8 +826,8 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                         const unsigned t = tag_of(l, 0);
                         if (q_sec >= 1) {
                             float* cr = pb.kv.pool + kv_at(l, q_sec - 1, p.gm.shard[g].head[q_hi], pos) + 2 * q_j;
-                            cr[0] = a;
-                            cr[1] = c;
+                            coherent_store(cr, a);
+                            coherent_store(cr + 1, c);
                         }
                         Cell* dst = p.xc + cl.qkv + (g * 2 + q_hi) * 192 + q_sec * 64 + 2 * q_j;
                         cell_put_local(dst, a, t);
@@ -755,36 +836,42 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 }
                 xcd_set_consumed(wt, wave, lane, unit_of(lay + me.o_wo));
             }
+            XTICK(0);
             stamp();
 
             // ===== P3: merge the slices' partials, W_o over this XCD's columns -> partial sums
             float bo_row = 0.0f;
             {
                 const int nap = SL * me.nh * kApCells;
-                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.ap + g * kApStrideCells, nap, tag_of(l, 1), apbuf, ctid, wt))
+                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.ap + g * kApStrideCells, nap, tag_of(l, 1), apbuf, ctid, wt, &stall[5]))
                     return;
-                if (!xcd_team_sync(wt, bar_gen, lane)) return;
+                XTICK(1);
+                if (!xcd_team_sync(wt, bar_gen, lane, &stall[9])) return;
+                XTICK(2);
                 stamp();
                 if (wave < kXcdRowWaves) {
-                    float* mine = att + wave * 128;
+                    float* mine = att + wave * (128 + 32);
+                    float* fw = mine + 128;  // [SL] this wavefront's merge factors
                     for (int hi = 0; hi < me.nh; hi++) {
+                        // slice q's (m, l) sit in lane q; one exponential per lane
                         const float* ap = apbuf + hi * SL * kApCells;
-                        float M = -INFINITY;
-                        for (int q = 0; q < SL; q++) M = fmaxf(M, ap[q * kApCells + 64]);
-                        float Ls = 0.0f, o = 0.0f;
-                        for (int q = 0; q < SL; q++) {
-                            const float f = expf(ap[q * kApCells + 64] - M);
-                            Ls += ap[q * kApCells + 65] * f;
-                            o += ap[q * kApCells + lane] * f;
-                        }
+                        const float mq = lane < SL ? ap[lane * kApCells + 64] : -INFINITY;
+                        const float lq = lane < SL ? ap[lane * kApCells + 65] : 0.0f;
+                        const float M = wave_max(mq);
+                        const float fq = expf(mq - M);  // 0 for empty slices and idle lanes
+                        const float Ls = wave_sum(lq * fq);
+                        if (lane < SL) fw[lane] = fq;
+                        lds_settle();
+                        float o = 0.0f;
+                        for (int q = 0; q < SL; q++) o += ap[q * kApCells + lane] * fw[q];
                         mine[hi * 64 + lane] = o * (1.0f / Ls);
+                        lds_settle();
                     }
-                    lds_settle();
                     const int sub = lane >> 4, dl = lane & 15;
                     const int nk4 = me.KC / 4;  // 16 or 32 float4 per row
                     for (int row = 4 * wave + sub; row < RW; row += 4 * kXcdRowWaves) {
                         const unsigned o = lay + me.o_wo + static_cast<unsigned>(row) * me.KC * 4u;
-                        if (!xcd_wait_filled(wt, units_to(lay + me.o_gu))) return;
+                        if (!xcd_wait_filled(wt, units_to(lay + me.o_gu), &stall[1])) return;
                         const unsigned base = unit_base * kXcdUnit + o;
                         float a = 0.0f;
                         for (int i = dl; i < nk4; i += 16)
@@ -801,6 +888,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 }
                 xcd_set_consumed(wt, wave, lane, unit_of(lay + me.o_gu));
             }
+            XTICK(3);
             stamp();
 
             // ===== P4: this workgroup's rows: the eight partials in XCD order + residual -> x'
@@ -811,6 +899,8 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                     make_buffer(p.xc + cl.part + which * kXcds * D, static_cast<unsigned>(kXcds * D) * 8u);
                 float pv[kXcds];
                 unsigned spins = 0;
+                XTICK(14);
+#pragma nounroll
                 for (;;) {
                     bool ok = true;
 #pragma unroll
@@ -828,6 +918,8 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                         return false;
                     }
                 }
+                XTICK(which);  // relay wavefront: 0 / 1 = time in the two polls, 14 = everything else
+                XROUNDS(2 + which, spins);
                 float sum = pv[0];
 #pragma unroll
                 for (int q = 1; q < kXcds; q++) sum += pv[q];
@@ -842,9 +934,11 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
 
             // ===== P5: norm2 + gate/up rows of this workgroup's hidden units -> hidden cells
             {
-                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (0 * kXcds + g) * D, D, tag_of(l, 3), xs1, ctid, wt))
+                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (0 * kXcds + g) * D, D, tag_of(l, 3), xs1, ctid, wt, &stall[6]))
                     return;
-                if (!xcd_team_sync(wt, bar_gen, lane)) return;
+                XTICK(4);
+                if (!xcd_team_sync(wt, bar_gen, lane, &stall[10])) return;
+                XTICK(5);
                 stamp();
                 float4 h[KD];
                 float ss = 0.0f;
@@ -857,7 +951,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 for (int k = wave; k < me.nu; k += kXcdTeamWaves) {
                     const unsigned o = lay + me.o_gu + static_cast<unsigned>(k) * 2u * D * 4u;
                     xcd_set_consumed(wt, wave, lane, unit_of(o));
-                    if (!xcd_wait_filled(wt, units_to(o + 2u * D * 4u))) return;
+                    if (!xcd_wait_filled(wt, units_to(o + 2u * D * 4u), &stall[2])) return;
                     const unsigned base = unit_base * kXcdUnit + o + lane * 16;
                     float a = 0.0f, c = 0.0f;
 #pragma unroll
@@ -873,20 +967,23 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 }
                 xcd_set_consumed(wt, wave, lane, unit_of(lay + me.o_dn));
             }
+            XTICK(6);
             stamp();
 
             // ===== P6: W_down over this XCD's hidden units -> partial sums
             {
-                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.hid + g * cl.hid_stride, me.UG, tag_of(l, 4), hbuf, ctid, wt))
+                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.hid + g * cl.hid_stride, me.UG, tag_of(l, 4), hbuf, ctid, wt, &stall[7], XTRIP(12)))
                     return;
-                if (!xcd_team_sync(wt, bar_gen, lane)) return;
+                XTICK(7);
+                if (!xcd_team_sync(wt, bar_gen, lane, &stall[11])) return;
+                XTICK(8);
                 stamp();
                 if (wave < kXcdRowWaves) {
                     const int sub = lane >> 4, dl = lane & 15;
                     const int nk4 = me.UG / 4;
                     for (int row = 4 * wave + sub; row < RW; row += 4 * kXcdRowWaves) {
                         const unsigned o = lay + me.o_dn + static_cast<unsigned>(row) * me.UG * 4u;
-                        if (!xcd_wait_filled(wt, units_to(lay + me.layer_bytes))) return;
+                        if (!xcd_wait_filled(wt, units_to(lay + me.layer_bytes), &stall[3])) return;
                         const unsigned base = unit_base * kXcdUnit + o;
                         float a = 0.0f;
                         for (int i = dl; i < nk4; i += 16)
@@ -897,14 +994,17 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 }
                 xcd_set_consumed(wt, wave, lane, unit_of(lay + me.layer_bytes));
             }
+            XTICK(9);
             stamp();
 
             // ===== P7: rows of this workgroup: partials + residual -> x of the next layer
             if (wave == kXcdRelayWave) {
                 if (!relay(1, xs1, 0.0f, 5, 6)) return;
             }
-            if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (1 * kXcds + g) * D, D, tag_of(l, 6), xs, ctid, wt)) return;
-            if (!xcd_team_sync(wt, bar_gen, lane)) return;
+            if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (1 * kXcds + g) * D, D, tag_of(l, 6), xs, ctid, wt, &stall[8], XTRIP(13))) return;
+            XTICK(10);
+            if (!xcd_team_sync(wt, bar_gen, lane, &stall[12])) return;
+            XTICK(11);
             stamp();
         }
         unit_base += me.layers_units;
@@ -923,7 +1023,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 const bool two = row + 1 < me.nrows;
                 const unsigned o = static_cast<unsigned>(row) * D * 4u;
                 xcd_set_consumed(wt, wave, lane, unit_base + (o >> 10));
-                if (!xcd_wait_filled(wt, unit_base + ((o + (two ? 2u : 1u) * D * 4u + 1023u) >> 10))) return;
+                if (!xcd_wait_filled(wt, unit_base + ((o + (two ? 2u : 1u) * D * 4u + 1023u) >> 10), &stall[4])) return;
                 const unsigned base = unit_base * kXcdUnit + o + lane * 16;
                 float a = 0.0f, c = 0.0f;
 #pragma unroll
@@ -956,7 +1056,21 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
         }
         stamp();
     }
-    if (!streamer && tid == 0) ctl[kXDone] = 1u;
+    if (!streamer && tid == 0) {
+        ctl[kXDone] = 1u;
+        if (pb.prof && wg == 0)
+            for (int i = 0; i < 13; i++) pb.prof[pb.prof_cap - 16 + i] = stall[i] + 1u;
+#ifdef GH_XCD_TICKS
+        if (pb.prof && wg == 0)
+            for (int i = 0; i < 16; i++) pb.prof[pb.prof_cap - 48 + i] = dur[i] + 1u;
+#endif
+    }
+#ifdef GH_XCD_TICKS
+    if (pb.prof && wg == 0 && lane == 0 && wave == kXcdRelayWave)
+        for (int i = 0; i < 16; i++) pb.prof[pb.prof_cap - 80 + i] = dur[i] + 1u;
+    if (pb.prof && wg == 0 && lane == 0 && wave == kXcdAttnWave)
+        for (int i = 0; i < 16; i++) pb.prof[pb.prof_cap - 112 + i] = dur[i] + 1u;
+#endif
 }
 
 }  // namespace gh

@@ -22,6 +22,7 @@ FLAG_PICK_GLOBAL_SCRATCH = 1
 FLAG_STEPWISE_PROMPT = 2
 FLAG_SMALL_ATTENTION_CHUNKS = 4
 FLAG_CLASSIC_PERSISTENT = 8
+FLAG_XCD_PERSISTENT = 16
 
 
 class DeviceError(RuntimeError):

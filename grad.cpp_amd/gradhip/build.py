@@ -16,7 +16,7 @@ LIB = os.path.join(LIB_DIR, "libgradhip.so")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-fno-fast-math", "-Wall", "-Wno-unused-function",
+    "-fno-fast-math", "-Wall", "-Wno-unused-function", *os.environ.get("GRADHIP_EXTRA_FLAGS", "").split(),
 ]
 SOURCES = ["engine.hip", "checkpoint.cpp", "tokenizer.cpp"]
 

@@ -120,10 +120,14 @@ enum { GH_FLAG_STEPWISE_PROMPT = 2 };
  * contexts. */
 enum { GH_FLAG_SMALL_ATTENTION_CHUNKS = 4 };
 
-/* Keep the persistent engine on its all-to-all kernel (every phase exchanged among
- * all 256 workgroups) where the XCD-sharded kernel would otherwise run; for
- * comparing the two and for testing the one that is not the default. */
+/* The persistent engine has two kernels for the Llama block at d_model 768: one in
+ * which every phase of a layer is exchanged among all 256 workgroups, and one that
+ * splits a layer over the eight XCDs and streams the weights through LDS.  By
+ * default a launch that starts at or beyond position 1536 takes the second (its
+ * attention is spread over all workgroups of an XCD) and every other launch the
+ * first.  These two flags pin the choice, for comparing the kernels and for tests. */
 enum { GH_FLAG_CLASSIC_PERSISTENT = 8 };
+enum { GH_FLAG_XCD_PERSISTENT = 16 };
 
 /* InferenceSession::InferenceSession (inference.cpp:121-148): allocates the
  * paged KV cache (2 * layers * max_len * d_model floats per sequence) and the
