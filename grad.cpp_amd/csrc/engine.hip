@@ -712,8 +712,11 @@ static PersistKernel persist_kernel_for(const Shape& sh, bool row_lds, bool feed
 
 // ---- the XCD-sharded form of the persistent kernel (kernels_xcd.h)
 
-// First position of a launch from which the XCD-sharded kernel is the default.
-constexpr int kXcdFromPosition = 1536;
+// First position of a launch from which the XCD-sharded kernel is the default.  Per
+// token on one box, Llama block d768 L8 V16000, greedy: positions 33..256 152 us against
+// 113 for the all-to-all kernel, 257..1024 184 / 154, 1024..1280 203 / 206, 1536..1792
+// 219 / 243, 2048..2304 235 / 281, 3072..3328 267 / 356.
+constexpr int kXcdFromPosition = 1024;
 
 using XcdKernel = void (*)(const XcdParams);
 

@@ -784,14 +784,17 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
     };
     if (coherent) {
         const __amdgpu_buffer_rsrc_t rs = make_buffer(logits, static_cast<unsigned>(V) * 4u);
-        // eight 16-byte loads per thread in flight; reads past the end return zero
-        bool counted = false;
-        for (int base = 4 * tid; base < V; base += 32 * nt) {
+        // eight 16-byte loads per thread in flight; reads past the end return zero.  The
+        // loop runs over rounds of the whole workgroup, so every wavefront is converged
+        // when wavefront 0 counts the window behind the first round of loads (the count
+        // reads other lanes' registers: with the loop bound depending on the thread, a
+        // vocabulary below four times the window left some of those lanes inactive).
+        for (int b0 = 0; b0 < V; b0 += 32 * nt) {
+            const int base = b0 + 4 * tid;
             v4i w[8];
 #pragma unroll
             for (int q = 0; q < 8; q++) w[q] = coherent_load16(rs, static_cast<unsigned>(base + q * 4 * nt) * 4u);
-            if (!counted) count_window();
-            counted = true;
+            if (b0 == 0) count_window();
 #pragma unroll
             for (int q = 0; q < 8; q++) {
                 const int i = base + q * 4 * nt;
@@ -806,7 +809,6 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
                 }
             }
         }
-        if (!counted) count_window();
     } else {
         row_pass(logits, V, [&](int i, float v) { val[i] = v; }, nt);
         count_window();

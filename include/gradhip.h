@@ -123,7 +123,7 @@ enum { GH_FLAG_SMALL_ATTENTION_CHUNKS = 4 };
 /* The persistent engine has two kernels for the Llama block at d_model 768: one in
  * which every phase of a layer is exchanged among all 256 workgroups, and one that
  * splits a layer over the eight XCDs and streams the weights through LDS.  By
- * default a launch that starts at or beyond position 1536 takes the second (its
+ * default a launch that starts at or beyond position 1024 takes the second (its
  * attention is spread over all workgroups of an XCD) and every other launch the
  * first.  These two flags pin the choice, for comparing the kernels and for tests. */
 enum { GH_FLAG_CLASSIC_PERSISTENT = 8 };

@@ -110,6 +110,29 @@ def test_long_context_runs_of_more_than_64_positions_per_wavefront():
             s.step([int(t)])
 
 
+def test_penalty_window_with_a_vocabulary_smaller_than_the_window_needs():
+    """The penalty window (50 tokens) is counted by one wavefront in registers.  With a
+    vocabulary of 100 fewer than 50 threads have a part of the row to load: the count must
+    not depend on that.  Tokens repeat all the time in so small a vocabulary, at every
+    window position."""
+    cfg = synth.Config(synth.ARCH_GPT2, 100, 512, 1, 8, 90)
+    W, om = make_pair(cfg, 31, std=0.05, norm_noise=0.1)
+    gm = G.Model.from_tensors(cfg, W)
+    prompt = synth.uniform_tokens(5, cfg.vocab, 3)
+    n = 80
+    u = synth.uniforms(n, 4)
+    for engine in (G.ENGINE_PERSISTENT, G.ENGINE_GRAPH):
+        s = G.Session(gm, engine=engine)
+        for penalty in (1.3, 0.8):
+            ref, rsl = O.generate_greedy(om, prompt, n, penalty, want_logits=True)
+            got = s.generate(prompt, n, G.sampling(greedy=True, repetition_penalty=penalty))
+            check_greedy_stream(got[0], ref, rsl, 5, f"vocab 100 greedy {penalty} engine {engine}")
+            opts = (0.9, 20, 0.9, penalty)
+            ref, rsl = O.generate_sample(om, prompt, u, opts[0], n, penalty, opts[1], opts[2], want_logits=True)
+            got = s.generate(prompt, n, G.sampling(*opts), uniforms=u)
+            check_sampled_stream(got[0], ref, rsl, 5, u, opts, f"vocab 100 sampled {penalty} engine {engine}")
+
+
 def test_unsupported_shapes_fall_back_or_refuse(models):
     cfg = synth.Config(synth.ARCH_MODERN, 301, 128, 2, 2, 40)
     gm = G.Model.from_tensors(cfg, synth.make_weights(cfg, 1))

@@ -128,28 +128,34 @@ def test_streaming_and_both_ways_of_ending_early(model):
 def test_long_context_and_the_default_choice_of_kernel():
     """Beyond 256 positions every workgroup of an XCD takes a slice of the attention, and
     beyond 32 positions per slice a slice is walked in several passes.  A session
-    without either flag runs launches that start at position 1536 or later on the
+    without either flag runs launches that start at position 1024 or later on the
     XCD kernel and the others on the all-to-all kernel; both must continue one
     context."""
-    cfg = synth.Config(synth.ARCH_MODERN, 500, 768, 1, 12, 1700)
+    cfg = synth.Config(synth.ARCH_MODERN, 500, 768, 1, 12, 1300)
     W, om = make_pair(cfg, 23, std=0.05, norm_noise=0.1)
     gm = G.Model.from_tensors(cfg, W)
     forced = G.Session(gm, engine=G.ENGINE_PERSISTENT, flags=XCD)
     auto = G.Session(gm, engine=G.ENGINE_PERSISTENT)
     osess = O.Session(om)
     toks = synth.uniform_tokens(cfg.max_len, cfg.vocab, 8)
-    for t in toks[:1500]:
+    for t in toks[:1000]:
         ref = osess.step(int(t))
-    assert_logits_close(forced.prefill(toks[None, :1500])[0], ref, 1e-4, "after a 1500-token prompt")
-    auto.prefill(toks[None, :1500])
-    for i, t in enumerate(toks[1500:]):
+    assert_logits_close(forced.prefill(toks[None, :1000])[0], ref, 1e-4, "after a 1000-token prompt")
+    auto.prefill(toks[None, :1000])
+    for i, t in enumerate(toks[1000:]):
         ref = osess.step(int(t))
         a = forced.step([int(t)])[0]
-        b = auto.step([int(t)])[0]
-        if i % 20 == 0 or i >= len(toks) - 1503:
-            assert_logits_close(a, ref, 1e-4, f"xcd position {1500 + i}")
-            assert_logits_close(b, ref, 1e-4, f"auto position {1500 + i}")
-        assert_logits_close(b, a, 2e-5)  # the cache rows of 1500..1535 came from two kernels: same up to sum order
+        b = auto.step([int(t)])[0]  # the all-to-all kernel up to position 1023, then the XCD kernel
+        if i % 20 == 0 or i >= len(toks) - 1003:
+            assert_logits_close(a, ref, 1e-4, f"xcd position {1000 + i}")
+            assert_logits_close(b, ref, 1e-4, f"auto position {1000 + i}")
+        assert_logits_close(b, a, 2e-5)  # some cache rows came from the other kernel: same up to sum order
+    # one launch that runs through the rest of a long context
+    s = G.Session(gm, engine=G.ENGINE_PERSISTENT, flags=XCD)
+    s.prefill(toks[None, :1100])
+    got = s.decode(150, G.sampling(greedy=True, repetition_penalty=1.0))[0]
+    ref, rsl = O.generate_greedy(om, toks[:1100], 150, 1.0, want_logits=True)
+    check_greedy_stream(np.concatenate([toks[:1100], got]), ref, rsl, 1100, "xcd long greedy run")
 
 
 def test_flags_exclude_each_other(model):
