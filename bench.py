@@ -40,6 +40,26 @@ PMC_WRITE_BYTES_PER_LAUNCH = 540_302 * 1024     # counter reads 1 per KiB writte
 PMC_ALGORITHMIC_BYTES_PER_LAUNCH = 63_406_751_744  # step_bytes() summed over that launch
 
 
+# Per-leg step times this tree is expected to reach on an MI355X (tracked next to the
+# profiles they come from); the line reports measured / expected for every leg, and
+# tests/test_gpu_regression.py fails beyond the file's tolerance.
+EXPECTED_FILE = os.path.join(ROOT, "profiles", "expected_step_times.json")
+
+
+def regression(line):
+    """{leg: measured ms per step / expected} for the legs of a bench line."""
+    try:
+        expected = json.load(open(EXPECTED_FILE))["ms_per_step"]
+    except (OSError, KeyError, ValueError):
+        return None
+    out = {}
+    for leg, want in expected.items():
+        got = line.get("ms_per_step") if leg == "c2" else (line.get(leg) or {}).get("ms_per_step")
+        if got and want:
+            out[leg] = round(got / want, 3)
+    return out
+
+
 def step_bytes(cfg, batch, ctx):
     """Algorithmic bytes of one decode step: every matrix once (regardless of
     batch), small vectors, the KV rows read at context `ctx` per sequence, the
@@ -52,10 +72,10 @@ def step_bytes(cfg, batch, ctx):
     return 4 * (mats + vecs + kv_read + batch * per_seq)
 
 
-def run_decode(G, synth, gm, cfg, batch, prompt_len, steps, warmup, opt, seed, engine):
+def run_decode(G, synth, gm, cfg, batch, prompt_len, steps, warmup, opt, seed, engine, flags=0):
     """Times exactly `steps` decode steps (in rounds that fit the context) with
     the host clock around synchronised GPU work; returns totals."""
-    gs = G.Session(gm, batch=batch, engine=engine)
+    gs = G.Session(gm, batch=batch, engine=engine, flags=flags)
     prompts = np.stack([synth.uniform_tokens(prompt_len, cfg.vocab, seed, stream=b) for b in range(batch)])
     room = cfg.max_len - prompt_len
     done = -warmup
@@ -173,10 +193,12 @@ def cpu_baseline(synth, W2):
             "single_thread": out["c2"]["threads_1"]["decode_tok_s"], "host_cpus": ncpu, "configs": out}
 
 
-def phase_stamps():
-    """Mean phase durations of one token of c2 on the persistent kernel, from the
-    stamps workgroup 0 leaves (GRADHIP_PROF_DUMP): per step one stamp after the pick,
-    five per layer, one when the logits rows have arrived, one at the end."""
+def phase_stamps(xcd=False):
+    """Mean phase durations of one token of c2 on a persistent kernel, from the stamps
+    workgroup 0 leaves (GRADHIP_PROF_DUMP).  The all-to-all kernel: per step one stamp
+    after the pick, five per layer, one when the logits rows have arrived, one at the
+    end.  The XCD-sharded kernel: one after the pick, eight per layer (a phase's
+    arithmetic, then the wait for the next phase's operands), one at the end."""
     import tempfile
     dump = os.path.join(tempfile.mkdtemp(), "stamps.txt")
     os.environ["GRADHIP_PROF_DUMP"] = dump
@@ -184,36 +206,52 @@ def phase_stamps():
     from gradhip import synth
     cfg = synth.PRESETS["c2"]
     gm = G.Model.from_tensors(cfg, synth.make_weights(cfg, 1002))
-    gs = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    gs = G.Session(gm, engine=G.ENGINE_PERSISTENT,
+                   flags=G.FLAG_XCD_PERSISTENT if xcd else G.FLAG_CLASSIC_PERSISTENT)
     gs.prefill(synth.uniform_tokens(32, cfg.vocab, 2002)[None, :])
     gs.decode(224, G.sampling(0.8, 40, 0.9, 1.1), seed=2002)
     gpu_us = gs.last_timing()["decode_ms"] * 1e3 / 224
-    gs.close()  # writes the dump
+    gs.close()  # writes the dump: stamps, "0", three clock readings per pick, "0", counters
     words = open(dump).read().split()
     z = words.index("0")
+    z2 = words.index("0", z + 1)
     st = np.array([int(x) for x in words[:z]], dtype=np.float64) / 100.0  # 100 MHz clock -> us
     L = cfg.layers
-    period = 5 * L + 3
+    per_layer = 8 if xcd else 5
+    period = per_layer * L + (2 if xcd else 3)
     d = np.diff(st)
     k = len(d) // period - 3
     m = d[2 * period: (2 + k) * period].reshape(k, period).mean(axis=0)
-    lay = m[1:1 + 5 * L].reshape(L, 5).mean(axis=0)
-    pk = np.array([int(x) for x in words[z + 1:]], dtype=np.float64) / 100.0
+    lay = m[1:1 + per_layer * L].reshape(L, per_layer).mean(axis=0)
+    pk = np.array([int(x) for x in words[z + 1:z2]], dtype=np.float64) / 100.0
     pk = pk[: len(pk) // 3 * 3].reshape(-1, 3)[3:]
-    print(json.dumps({
+    out = {
         "workload": "c2, one launch of 224 pick + step rounds, contexts 33..256", "steps_averaged": int(k),
+        "kernel": "xcd_decode_kernel" if xcd else "persist_decode_kernel",
         "us_per_token_events": round(gpu_us, 2), "us_per_token_stamps": round(float(m.sum()), 2),
         "pick_until_token_seen": round(float(m[0]), 2),
         "pick_inside": {"wait_for_logits": round(float((pk[:, 1] - pk[:, 0]).mean()), 2),
-                        "penalty_sampler_token_out": round(float((pk[:, 2] - pk[:, 1]).mean()), 2)},
-        "layer_mean": {"embed_or_x_exchange+norm1+qkv": round(float(lay[0]), 2),
-                       "qkv_exchange+attention": round(float(lay[1]), 2),
-                       "attn_exchange+w_o": round(float(lay[2]), 2),
-                       "x_exchange+norm2+ffn1": round(float(lay[3]), 2),
-                       "hidden_exchange+ffn2": round(float(lay[4]), 2), "sum": round(float(lay.sum()), 2)},
-        "layers_total": round(float(lay.sum() * L), 2),
-        "x_exchange+logits_rows_arrive": round(float(m[-2]), 2),
-        "logits_dots_stores_arrival_count": round(float(m[-1]), 2)}))
+                        "penalty_sampler_token_out": round(float((pk[:, 2] - pk[:, 1]).mean()), 2)}}
+    if xcd:
+        names = ["norm1+qkv_rows", "wait_attention_partials", "merge+w_o_partials", "wait_x_after_attention",
+                 "norm2+gate_up_rows", "wait_hidden", "w_down_partials", "wait_x_of_next_layer"]
+        out["layer_mean"] = {n: round(float(v), 2) for n, v in zip(names, lay)}
+        out["layer_mean"]["sum"] = round(float(lay.sum()), 2)
+        out["layers_total"] = round(float(lay.sum() * L), 2)
+        out["logits_rows_from_the_ring"] = round(float(m[-1]), 2)
+        tail = [int(x) for x in words[z2 + 1:]]
+        # polls that found the ring not yet filled, per token (stored + 1): P1, P3, P5, P6, logits
+        out["ring_stall_polls_per_token"] = [round((v - 1) / 224.0, 2) for v in tail[96:101] if v > 0]
+    else:
+        out["layer_mean"] = {"embed_or_x_exchange+norm1+qkv": round(float(lay[0]), 2),
+                             "qkv_exchange+attention": round(float(lay[1]), 2),
+                             "attn_exchange+w_o": round(float(lay[2]), 2),
+                             "x_exchange+norm2+ffn1": round(float(lay[3]), 2),
+                             "hidden_exchange+ffn2": round(float(lay[4]), 2), "sum": round(float(lay.sum()), 2)}
+        out["layers_total"] = round(float(lay.sum() * L), 2)
+        out["x_exchange+logits_rows_arrive"] = round(float(m[-2]), 2)
+        out["logits_dots_stores_arrival_count"] = round(float(m[-1]), 2)
+    print(json.dumps(out))
 
 
 def main():
@@ -243,9 +281,11 @@ def main():
                     help="only run one 224-step launch of the batch-1 workload with the persistent kernel's "
                          "in-kernel phase stamps on (workgroup 0's clock at the end of every phase) and "
                          "print the mean duration of every phase of a token")
+    ap.add_argument("--phase-stamps-xcd", action="store_true",
+                    help="the same for the XCD-sharded persistent kernel (eight stamps per layer)")
     a = ap.parse_args()
-    if a.phase_stamps:
-        phase_stamps()
+    if a.phase_stamps or a.phase_stamps_xcd:
+        phase_stamps(xcd=a.phase_stamps_xcd)
         return
     if a.cache_probe:
         import gradhip as G
@@ -335,8 +375,8 @@ def main():
                           " of its algorithmic bytes; scaled to this launch's algorithmic bytes")
     else:
         kernel = "every kernel of the decode round (one launch per fused op), timed as one span"
-        traffic = int(bytes_per_launch)
-        traffic_source = "algorithmic bytes (no counter run covers this engine)"
+        traffic = None
+        traffic_source = "no counter run covers this engine"
 
     line = {
         "metric": "decode tok/s, 69M Llama block, batch 1",
@@ -350,6 +390,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "traffic_source": traffic_source,
+                     "traffic_is": "this launch's algorithmic bytes times the HBM-to-algorithmic ratio that "
+                                   "rocprofv3 --pmc measured on a 224-step launch of the same kernel; not "
+                                   "re-measured in this run" if traffic is not None else None,
                      "kernel": kernel, "launches": n_l, "steps_per_launch": steps_per_launch,
                      "us_per_launch": round(us_per_launch, 1),
                      "bytes_per_launch": int(bytes_per_launch)},
@@ -381,6 +424,42 @@ def main():
                          "224 greedy steps", r1m, 1)
         del gm1
 
+    if not a.no_small:
+        # The reference's own published protocol for this path (src/cli/bench.cpp:269-286):
+        # five timed calls of generate_sample(prompt, temperature 0.8, 64 tokens) with
+        # TextGen's defaults (penalty 1.2, no top-k / top-p) on the 'small' GPT-2 shape with
+        # the presets' context of 1024, a fresh session per call, host wall time including
+        # the session's construction and the prompt steps; median of 64 / seconds.  Its
+        # published figures: 385.1 tok/s (M2 Pro), 843.5 / 854.5 (M3 Pro).
+        cfgb = synth.Config(synth.ARCH_GPT2, 5000, 512, 6, 8, 1024)
+        gmb = G.Model.from_tensors(cfgb, synth.make_weights(cfgb, 1000))
+        prompt_b = np.frombuffer(b"ROMEO:\n", dtype=np.uint8).astype(np.int32)[None, :]
+        rates = []
+        for trial in range(6):
+            t0 = time.perf_counter()
+            sb = G.Session(gmb)
+            toks = sb.generate(prompt_b, 64, G.sampling(0.8, 0, 1.0, 1.2), seed=trial)
+            sb.close()
+            dt = time.perf_counter() - t0
+            assert toks.shape[1] == prompt_b.shape[1] + 64
+            if trial:  # the first call also loads the kernels' code: a warm-up, like a first run of the binary
+                rates.append(64.0 / dt)
+        line["grad_bench_protocol"] = {
+            "workload": "grad bench's generation figure: GPT-2 'small' (d512 L6 H8 V5000 C1024), 7-token prompt, "
+                        "generate_sample(T 0.8, 64 tokens, penalty 1.2), fresh session per call, wall time "
+                        "including session construction; median of 5 calls after one warm-up call",
+            "value": round(float(np.median(rates)), 1), "unit": "tok/s", "trials": [round(r, 1) for r in rates],
+            "reference_published": {"M2 Pro": 385.1, "M3 Pro": [843.5, 854.5]}}
+        del gmb
+        # Batch 1 at the context every preset of the reference ships (max_len 1024): the c2
+        # weights, a 256-token prompt, greedy to the end of the context.
+        cfgl = synth.Config(cfg.arch, cfg.vocab, cfg.d_model, cfg.layers, cfg.heads, 1024)
+        gml = G.Model.from_tensors(cfgl, W)
+        rl = run_decode(G, synth, gml, cfgl, 1, 256, 768, 768, greedy, 2002, engine)
+        line["c2_ctx1024"] = leg("c2 weights with max_len 1024 (the reference presets' context), batch 1, "
+                                 "256-token prompt, 768 greedy steps to the end of the context", rl, 1)
+        del gml
+
     if not a.no_batch64:
         r64 = run_decode(G, synth, gm, cfg, 64, 128, 128, 16, greedy, 2003, engine)
         line["batch64"] = leg("c3: same model, 64 sequences, 128-token prompts, 128 greedy steps", r64, 64)
@@ -395,6 +474,7 @@ def main():
                                   "in one pass, 512 greedy steps", r4, 16)
         del gm4
 
+    line["regression"] = regression(line)
     line["cpu_baseline"] = None if a.no_cpu else cpu_baseline(synth, W)
     print(json.dumps(line), flush=True)
 

@@ -1181,11 +1181,16 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
                 // Test aid: start the session's two running counts `near` steps before the
                 // points where the arrival counters wrap around 2^32 and where the cell tags
                 // are re-based, so that a short run crosses both.
-                const unsigned n = static_cast<unsigned>(std::atoi(near));
-                s.arrive_total = (0u - n * static_cast<unsigned>(s.persist_grid)) / static_cast<unsigned>(s.persist_grid);
-                const unsigned sum = s.arrive_total * static_cast<unsigned>(s.persist_grid);
-                HIP_CHECK(hipMemcpy(&s.ctl->arrive[0], &sum, sizeof(sum), hipMemcpyHostToDevice));
-                s.epoch = static_cast<unsigned>(0xF0000000ull / (static_cast<unsigned long long>(sh.layers + 1) * 8ull)) - n;
+                // (a test hook: values outside 1..4096 are ignored, so a stray variable cannot
+                // leave the counters inconsistent)
+                const long asked = std::strtol(near, nullptr, 10);
+                const unsigned n = asked >= 1 && asked <= 4096 ? static_cast<unsigned>(asked) : 0u;
+                if (n != 0u) {
+                    s.arrive_total = (0u - n * static_cast<unsigned>(s.persist_grid)) / static_cast<unsigned>(s.persist_grid);
+                    const unsigned sum = s.arrive_total * static_cast<unsigned>(s.persist_grid);
+                    HIP_CHECK(hipMemcpy(&s.ctl->arrive[0], &sum, sizeof(sum), hipMemcpyHostToDevice));
+                    s.epoch = static_cast<unsigned>(0xF0000000ull / (static_cast<unsigned long long>(sh.layers + 1) * 8ull)) - n;
+                }
             }
             if (std::getenv("GRADHIP_PROF_DUMP")) {
                 s.prof_cap = 1 << 16;

@@ -815,7 +815,9 @@ __device__ __forceinline__ int pick_body(const PickParams& p, int b, float* val,
     }
     __syncthreads();
     if (p.penalty != 1.0f) {
-        if (pen_first) {
+        // ids come from the session's own history, or from the caller's device memory in the
+        // entry point that allocates nothing: one outside the vocabulary is left alone
+        if (pen_first && static_cast<unsigned>(window_token) < static_cast<unsigned>(V)) {
             float v = val[window_token];
             for (int c = 0; c < pen_times; c++) v = (v > 0.0f) ? v / p.penalty : v * p.penalty;
             val[window_token] = v;
