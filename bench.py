@@ -281,6 +281,13 @@ def main():
                     help="only run one 224-step launch of the batch-1 workload with the persistent kernel's "
                          "in-kernel phase stamps on (workgroup 0's clock at the end of every phase) and "
                          "print the mean duration of every phase of a token")
+    ap.add_argument("--kernel", default="auto", choices=["auto", "classic", "xcd"],
+                    help="pin the batch-1 legs to one of the persistent engine's two kernels (the all-to-all "
+                         "kernel or the XCD-sharded one); auto: by position, as sessions do by default")
+    ap.add_argument("--step-loop", action="store_true",
+                    help="only time the literal drop-in loop on the batch-1 workload: one InferenceSession::step "
+                         "call per token (one launch and one copy of the logits to the host each) with the "
+                         "arg-max on the host, as text_gen.cpp:44-64 does, and exit")
     ap.add_argument("--phase-stamps-xcd", action="store_true",
                     help="the same for the XCD-sharded persistent kernel (eight stamps per layer)")
     a = ap.parse_args()
@@ -328,6 +335,24 @@ def main():
     opts = (0.8, 40, 0.9, 1.1)
     sample = G.sampling(*opts)
 
+    b1_flags = {"auto": 0, "classic": G.FLAG_CLASSIC_PERSISTENT, "xcd": G.FLAG_XCD_PERSISTENT}[a.kernel]
+    if a.step_loop:
+        gs = G.Session(gm, engine=engine, flags=b1_flags)
+        prompt = synth.uniform_tokens(32, cfg.vocab, 2002)
+        best = None
+        for rep in range(3):
+            gs.reset()
+            logits = gs.prefill(prompt[None, :])[0]
+            t0 = time.perf_counter()
+            for _ in range(224):
+                logits = gs.step([int(np.argmax(logits))])[0]
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        print(json.dumps({"workload": "c2, 32-token prompt, 224 x (host arg-max + step() with the logits copied "
+                                      "to the host)", "value": round(224 / best, 1), "unit": "tok/s",
+                          "us_per_token": round(best * 1e6 / 224, 2), "kernel": a.kernel,
+                          "launches_per_step": gs.last_timing()["launches_per_step"]}), flush=True)
+        return
     if a.only_batch64:
         greedy = G.sampling(greedy=True, repetition_penalty=1.0)
         r64 = run_decode(G, synth, gm, cfg, 64, 128, 128, 16, greedy, 2003, engine)
@@ -353,7 +378,7 @@ def main():
                 "ms_per_step": round(r["wall_s"] * 1e3 / r["steps"], 5),
                 "prefill_tok_s": round(r["prefill_tok_s"], 1), "roofline": roofline(r)}
 
-    r1 = run_decode(G, synth, gm, cfg, 1, 32, a.steps, a.warmup, sample, 2002, engine)
+    r1 = run_decode(G, synth, gm, cfg, 1, 32, a.steps, a.warmup, sample, 2002, engine, b1_flags)
     tok_s = r1["steps"] / r1["wall_s"]
     persistent = r1["launches_per_step"] == 1
     n_l = len(r1["launches"])
@@ -367,6 +392,9 @@ def main():
         kernel = (f"gh::persist_decode_kernel<{cfg.d_model // 256}, {cfg.d_ff // 256}, "
                   f"{'true' if cfg.modern else 'false'}, {'true' if cfg.vocab <= 38000 else 'false'}, false>: "
                   "one launch = one pick + step round per token for a whole run of steps")
+        if a.kernel == "xcd":
+            kernel = ("gh::xcd_decode_kernel<3, true, false>: the XCD-sharded persistent kernel, one launch = one "
+                      "pick + step round per token for a whole run of steps")
         # measured HBM bytes per algorithmic byte of this kernel, times this launch's algorithmic bytes
         traffic = int(bytes_per_launch * (PMC_FETCH_BYTES_PER_LAUNCH + PMC_WRITE_BYTES_PER_LAUNCH)
                       / PMC_ALGORITHMIC_BYTES_PER_LAUNCH)
@@ -407,7 +435,7 @@ def main():
     greedy = G.sampling(greedy=True, repetition_penalty=1.0)
     if not a.no_small:
         # the workload exactly as named, whatever --steps says: 32 prompt tokens, 224 sampled steps
-        rf = run_decode(G, synth, gm, cfg, 1, 32, 224, 224, sample, 2002, engine)
+        rf = run_decode(G, synth, gm, cfg, 1, 32, 224, 224, sample, 2002, engine, b1_flags)
         line["c2_full"] = leg("c2 as named: 32-token prompt, then 224 sampled decode steps (one launch)", rf, 1)
         # c0 (the shape of the reference's own published figure) and c1
         cfg0 = synth.PRESETS["c0"]
@@ -455,7 +483,7 @@ def main():
         # weights, a 256-token prompt, greedy to the end of the context.
         cfgl = synth.Config(cfg.arch, cfg.vocab, cfg.d_model, cfg.layers, cfg.heads, 1024)
         gml = G.Model.from_tensors(cfgl, W)
-        rl = run_decode(G, synth, gml, cfgl, 1, 256, 768, 768, greedy, 2002, engine)
+        rl = run_decode(G, synth, gml, cfgl, 1, 256, 768, 768, greedy, 2002, engine, b1_flags)
         line["c2_ctx1024"] = leg("c2 weights with max_len 1024 (the reference presets' context), batch 1, "
                                  "256-token prompt, 768 greedy steps to the end of the context", rl, 1)
         del gml

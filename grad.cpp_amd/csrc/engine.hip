@@ -893,7 +893,7 @@ static const char* persist_unavailable(const Session& s, int lds_bytes, int cus)
 // stop word and stop_token.
 static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool start_with_pick,
                         const gh_sampling* o, const float* dev_uniforms, int u_stride, uint64_t seed,
-                        float* logit_log, bool feed = false, int stop_token = -1) {
+                        float* logit_log, bool feed = false, int stop_token = -1, int tok0 = -1) {
     const Model& m = *s.m;
     const Shape& sh = m.shape;
     if (n_steps <= 0 && n_picks <= 0) return;
@@ -934,6 +934,7 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     p.n_steps = n_steps;
     p.n_picks = n_picks;
     p.start_with_pick = start_with_pick ? 1 : 0;
+    p.tok0 = tok0;
     p.epoch = s.epoch;
     p.arrive_base = s.arrive_total;
     p.spin_limit = 1u << 18;
@@ -1946,23 +1947,33 @@ gh_status gh_session_step(gh_session* sess, const int32_t* ids, float* logits_ho
         check_capacity(s);
         check_ids(s, ids, s.B);
         const size_t V = s.m->shape.vocab;
-        std::memcpy(s.host_ids, ids, s.B * sizeof(int));
-        HIP_CHECK(hipMemcpyAsync(s.tok, s.host_ids, s.B * sizeof(int), hipMemcpyHostToDevice,
-                                 s.stream));
-        // The history (index == position) feeds the repetition penalty of later picks.
-        hipLaunchKernelGGL(store_hist_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
-                           s.hist_stride, s.n_hist, s.tok, s.B);
-        HIP_CHECK(hipGetLastError());
-        if (s.engine == GH_ENGINE_PERSISTENT) {
-            persist_run(s, 1, 1, 0, false, nullptr, nullptr, 0, 0, nullptr);
+        const bool one_launch = s.engine == GH_ENGINE_PERSISTENT && s.n_hist == s.pos;
+        if (one_launch) {
+            // One launch, one copy back and one wait per call: the token travels in the
+            // kernel's arguments (the kernel records it in the history, whose index is the
+            // position), and the kernel's "gave up" word comes back with the logits.
+            persist_run(s, 1, 1, 0, false, nullptr, nullptr, 0, 0, nullptr, false, -1, ids[0]);
+            HIP_CHECK(hipMemcpyAsync(s.host_err, &s.ctl->abort, sizeof(int), hipMemcpyDeviceToHost, s.stream));
         } else {
-            s.n_hist++;
-            run_step(s);
+            std::memcpy(s.host_ids, ids, s.B * sizeof(int));
+            HIP_CHECK(hipMemcpyAsync(s.tok, s.host_ids, s.B * sizeof(int), hipMemcpyHostToDevice,
+                                     s.stream));
+            // The history (index == position) feeds the repetition penalty of later picks.
+            hipLaunchKernelGGL(store_hist_kernel, dim3((s.B + 63) / 64), dim3(64), 0, s.stream, s.hist,
+                               s.hist_stride, s.n_hist, s.tok, s.B);
+            HIP_CHECK(hipGetLastError());
+            if (s.engine == GH_ENGINE_PERSISTENT) {
+                persist_run(s, 1, 1, 0, false, nullptr, nullptr, 0, 0, nullptr);
+            } else {
+                s.n_hist++;
+                run_step(s);
+            }
         }
         HIP_CHECK(hipMemcpyAsync(s.host_logits, s.logits, s.B * V * sizeof(float),
                                  hipMemcpyDeviceToHost, s.stream));
         HIP_CHECK(hipStreamSynchronize(s.stream));
-        check_persist_abort(s);
+        // (the word read back with the logits says whether the kernel finished its waits)
+        if (!one_launch || *s.host_err != 0) check_persist_abort(s);
         if (logits_host) std::memcpy(logits_host, s.host_logits, s.B * V * sizeof(float));
     });
 }

@@ -98,6 +98,7 @@ struct PersistParams {
     int n_steps;       // step() calls in this launch
     int n_picks;       // picks in this launch
     int start_with_pick;  // the first pick uses the logits already in memory
+    int tok0;             // >= 0: the token of step 0 (not yet in the history: the kernel records it)
     unsigned epoch;    // tag base of this launch; (epoch + s) never repeats in a session
     unsigned arrive_base;  // logits phases completed before this launch
     PickParams pick;
@@ -461,7 +462,14 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         // ---- token and embedding (inference.cpp:159-182)
         int tok;
         if (s < p.n_prompt) {
-            tok = p.hist[pos];
+            if (s == 0 && p.tok0 >= 0) {
+                // handed over in the launch's arguments: no copy and no launch in front of a single step
+                tok = p.tok0;
+                if (wg == 0 && tid == 0)
+                    __hip_atomic_store(&p.hist[pos], tok, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                tok = p.hist[pos];
+            }
         } else {
             // the pick that followed step s-1 (or opened the launch)
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)

@@ -56,7 +56,7 @@ constexpr int kXcdRelayWave = 6;      // sums the partials of this workgroup's r
 constexpr int kXcdAttnWave = 7;       // attention of one slice (P2); takes no part in anything else
 constexpr int kXcds = 8, kWgPerXcd = 32;
 constexpr int kXcdUnit = 1024;        // bytes one streamer instruction moves
-constexpr int kXcdDepth = 8;          // loads a streamer keeps in flight
+constexpr int kXcdDepth = 16;         // loads a streamer keeps in flight
 constexpr int kAuxNonTemporal = 2;    // nt on gfx94x / gfx950 buffer instructions
 constexpr int kApCells = 66;          // cells of one attention partial: acc[64], m, l
 constexpr int kXcdMaxUnitsPerWg = 2 * kXcdTeamWaves;
@@ -522,8 +522,13 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
     int i_pick = 0;
     unsigned arrive_gen = pb.arrive_base;
     bool ended = false;
-    unsigned stall[13] = {};
+    // Diagnostics, compiled in with -DGH_XCD_TICKS only (the counters cost registers the
+    // kernel does not have to spare): polls that found the ring not yet filled and poll
+    // rounds of the gathers, per phase, and the core clock spent in every phase by
+    // wavefront 0, the relay wavefront and the attention wavefront of workgroup 0.
 #ifdef GH_XCD_TICKS
+    unsigned stall[13] = {};
+#define XSTALL(k) (&stall[k])
     unsigned dur[16] = {};
     unsigned last_tick = 0;
 #define XTICK(k)                                                                  \
@@ -535,10 +540,11 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
 #define XTRIP(k) (&dur[k])
 #define XROUNDS(k, n) dur[k] += (n)
 #else
+#define XSTALL(k) nullptr
 #define XROUNDS(k, n) do { } while (0)
 #define XTICK(k) do { } while (0)
 #define XTRIP(k) nullptr
-#endif  // polls spent waiting for the ring, by phase (diagnostics)
+#endif
     int n_stamp = 0;
     auto stamp = [&]() {
         if (pb.prof && wg == 0 && tid == 0 && n_stamp < pb.prof_cap / 2) pb.prof[n_stamp] = __builtin_amdgcn_s_memrealtime();
@@ -598,7 +604,13 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
         // ---- token (inference.cpp:159-182): every wavefront reads it for itself
         int tok;
         if (s < pb.n_prompt) {
-            tok = pb.hist[pos];
+            if (s == 0 && pb.tok0 >= 0) {
+                tok = pb.tok0;  // handed over in the launch's arguments
+                if (wg == 0 && tid == 0)
+                    __hip_atomic_store(&pb.hist[pos], tok, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                tok = pb.hist[pos];
+            }
         } else {
             const unsigned tt = ((pb.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
@@ -802,7 +814,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 if (wave < me.ppw) {
                     const unsigned o = lay + static_cast<unsigned>(wave) * me.pair_bytes;
                     xcd_set_consumed(wt, wave, lane, unit_of(o));
-                    if (!xcd_wait_filled(wt, units_to(o + me.pair_bytes), &stall[0])) return;
+                    if (!xcd_wait_filled(wt, units_to(o + me.pair_bytes), XSTALL(0))) return;
                     const float rn = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(D) + kNormEps);
                     float a = 0.0f, c = 0.0f;
                     const unsigned base = unit_base * kXcdUnit + o + lane * 16;
@@ -843,10 +855,10 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
             float bo_row = 0.0f;
             {
                 const int nap = SL * me.nh * kApCells;
-                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.ap + g * kApStrideCells, nap, tag_of(l, 1), apbuf, ctid, wt, &stall[5]))
+                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.ap + g * kApStrideCells, nap, tag_of(l, 1), apbuf, ctid, wt, XSTALL(5)))
                     return;
                 XTICK(1);
-                if (!xcd_team_sync(wt, bar_gen, lane, &stall[9])) return;
+                if (!xcd_team_sync(wt, bar_gen, lane, XSTALL(9))) return;
                 XTICK(2);
                 stamp();
                 if (wave < kXcdRowWaves) {
@@ -871,7 +883,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                     const int nk4 = me.KC / 4;  // 16 or 32 float4 per row
                     for (int row = 4 * wave + sub; row < RW; row += 4 * kXcdRowWaves) {
                         const unsigned o = lay + me.o_wo + static_cast<unsigned>(row) * me.KC * 4u;
-                        if (!xcd_wait_filled(wt, units_to(lay + me.o_gu), &stall[1])) return;
+                        if (!xcd_wait_filled(wt, units_to(lay + me.o_gu), XSTALL(1))) return;
                         const unsigned base = unit_base * kXcdUnit + o;
                         float a = 0.0f;
                         for (int i = dl; i < nk4; i += 16)
@@ -934,10 +946,10 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
 
             // ===== P5: norm2 + gate/up rows of this workgroup's hidden units -> hidden cells
             {
-                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (0 * kXcds + g) * D, D, tag_of(l, 3), xs1, ctid, wt, &stall[6]))
+                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (0 * kXcds + g) * D, D, tag_of(l, 3), xs1, ctid, wt, XSTALL(6)))
                     return;
                 XTICK(4);
-                if (!xcd_team_sync(wt, bar_gen, lane, &stall[10])) return;
+                if (!xcd_team_sync(wt, bar_gen, lane, XSTALL(10))) return;
                 XTICK(5);
                 stamp();
                 float4 h[KD];
@@ -951,7 +963,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 for (int k = wave; k < me.nu; k += kXcdTeamWaves) {
                     const unsigned o = lay + me.o_gu + static_cast<unsigned>(k) * 2u * D * 4u;
                     xcd_set_consumed(wt, wave, lane, unit_of(o));
-                    if (!xcd_wait_filled(wt, units_to(o + 2u * D * 4u), &stall[2])) return;
+                    if (!xcd_wait_filled(wt, units_to(o + 2u * D * 4u), XSTALL(2))) return;
                     const unsigned base = unit_base * kXcdUnit + o + lane * 16;
                     float a = 0.0f, c = 0.0f;
 #pragma unroll
@@ -972,10 +984,10 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
 
             // ===== P6: W_down over this XCD's hidden units -> partial sums
             {
-                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.hid + g * cl.hid_stride, me.UG, tag_of(l, 4), hbuf, ctid, wt, &stall[7], XTRIP(12)))
+                if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.hid + g * cl.hid_stride, me.UG, tag_of(l, 4), hbuf, ctid, wt, XSTALL(7), XTRIP(12)))
                     return;
                 XTICK(7);
-                if (!xcd_team_sync(wt, bar_gen, lane, &stall[11])) return;
+                if (!xcd_team_sync(wt, bar_gen, lane, XSTALL(11))) return;
                 XTICK(8);
                 stamp();
                 if (wave < kXcdRowWaves) {
@@ -983,7 +995,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                     const int nk4 = me.UG / 4;
                     for (int row = 4 * wave + sub; row < RW; row += 4 * kXcdRowWaves) {
                         const unsigned o = lay + me.o_dn + static_cast<unsigned>(row) * me.UG * 4u;
-                        if (!xcd_wait_filled(wt, units_to(lay + me.layer_bytes), &stall[3])) return;
+                        if (!xcd_wait_filled(wt, units_to(lay + me.layer_bytes), XSTALL(3))) return;
                         const unsigned base = unit_base * kXcdUnit + o;
                         float a = 0.0f;
                         for (int i = dl; i < nk4; i += 16)
@@ -1001,9 +1013,9 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
             if (wave == kXcdRelayWave) {
                 if (!relay(1, xs1, 0.0f, 5, 6)) return;
             }
-            if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (1 * kXcds + g) * D, D, tag_of(l, 6), xs, ctid, wt, &stall[8], XTRIP(13))) return;
+            if (!xcd_gather<kAuxNonTemporal>(p.xc + cl.xr + (1 * kXcds + g) * D, D, tag_of(l, 6), xs, ctid, wt, XSTALL(8), XTRIP(13))) return;
             XTICK(10);
-            if (!xcd_team_sync(wt, bar_gen, lane, &stall[12])) return;
+            if (!xcd_team_sync(wt, bar_gen, lane, XSTALL(12))) return;
             XTICK(11);
             stamp();
         }
@@ -1023,7 +1035,7 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
                 const bool two = row + 1 < me.nrows;
                 const unsigned o = static_cast<unsigned>(row) * D * 4u;
                 xcd_set_consumed(wt, wave, lane, unit_base + (o >> 10));
-                if (!xcd_wait_filled(wt, unit_base + ((o + (two ? 2u : 1u) * D * 4u + 1023u) >> 10), &stall[4])) return;
+                if (!xcd_wait_filled(wt, unit_base + ((o + (two ? 2u : 1u) * D * 4u + 1023u) >> 10), XSTALL(4))) return;
                 const unsigned base = unit_base * kXcdUnit + o + lane * 16;
                 float a = 0.0f, c = 0.0f;
 #pragma unroll
@@ -1058,11 +1070,11 @@ __global__ __launch_bounds__(kXcdThreads) void xcd_decode_kernel(const XcdParams
     }
     if (!streamer && tid == 0) {
         ctl[kXDone] = 1u;
-        if (pb.prof && wg == 0)
-            for (int i = 0; i < 13; i++) pb.prof[pb.prof_cap - 16 + i] = stall[i] + 1u;
 #ifdef GH_XCD_TICKS
-        if (pb.prof && wg == 0)
+        if (pb.prof && wg == 0) {
+            for (int i = 0; i < 13; i++) pb.prof[pb.prof_cap - 16 + i] = stall[i] + 1u;
             for (int i = 0; i < 16; i++) pb.prof[pb.prof_cap - 48 + i] = dur[i] + 1u;
+        }
 #endif
     }
 #ifdef GH_XCD_TICKS
