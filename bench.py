@@ -288,11 +288,28 @@ def main():
                     help="only time the literal drop-in loop on the batch-1 workload: one InferenceSession::step "
                          "call per token (one launch and one copy of the logits to the host each) with the "
                          "arg-max on the host, as text_gen.cpp:44-64 does, and exit")
+    ap.add_argument("--handoff-probe", action="store_true",
+                    help="only time a two-workgroup ping-pong (same XCD / two XCDs, ordinary or device-scope "
+                         "stores, non-temporal or device-scope loads, idle or beside 240 streaming workgroups) "
+                         "and exit")
     ap.add_argument("--phase-stamps-xcd", action="store_true",
                     help="the same for the XCD-sharded persistent kernel (eight stamps per layer)")
     a = ap.parse_args()
     if a.phase_stamps or a.phase_stamps_xcd:
         phase_stamps(xcd=a.phase_stamps_xcd)
+        return
+    if a.handoff_probe:
+        import gradhip as G
+        rows = []
+        for busy in (False, True):
+            for peer in (8, 1):
+                for store_dev, load, name in ((True, 2, "device-scope store, device-scope load"),
+                                              (True, 1, "device-scope store, non-temporal load"),
+                                              (False, 1, "ordinary store, non-temporal load"),
+                                              (False, 2, "ordinary store, device-scope load")):
+                    us, xa, xb = G.handoff_latency(load, store_dev, peer, busy)
+                    rows.append({"busy": busy, "xcds": [xa, xb], "policy": name, "us_per_round_trip": round(us, 3)})
+        print(json.dumps({"handoff": rows}))
         return
     if a.cache_probe:
         import gradhip as G

@@ -1651,6 +1651,60 @@ static float* scratch_on_current_device() {
     return g_scratch_ptr[dev];
 }
 
+// ---- hand-off latency probe (gh_device_handoff_latency)
+
+// Workgroup 0 and workgroup `peer` bounce a counter: each waits until the other's word
+// has reached the round number and then writes its own.  LOAD: cache policy of the
+// polling load (buffer aux bits); DEVICE_STORE: device-scope (write-through) store or
+// an ordinary one.  Bounded polling: a side that never sees its peer gives up.
+template <int LOAD, bool DEVICE_STORE>
+__global__ void handoff_probe_kernel(unsigned* cells, int peer, int rounds, unsigned long long* ticks, unsigned* xcds) {
+    const int me = blockIdx.x == 0 ? 0 : (static_cast<int>(blockIdx.x) == peer ? 1 : -1);
+    if (threadIdx.x == 0) xcds[blockIdx.x] = xcc_id();
+    if (me < 0 || threadIdx.x != 0) return;
+    unsigned* mine = cells + me * 64;
+    const __amdgpu_buffer_rsrc_t rs = make_buffer(cells + (1 - me) * 64, 4);
+    auto put = [&](unsigned v) {
+        if (DEVICE_STORE) __hip_atomic_store(mine, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else *reinterpret_cast<volatile unsigned*>(mine) = v;
+    };
+    const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+    for (int i = 1; i <= rounds; i++) {
+        if (me == 0) put(static_cast<unsigned>(i));
+        unsigned spins = 0;
+        while (static_cast<unsigned>(__builtin_amdgcn_raw_buffer_load_b32(rs, 0, 0, LOAD)) < static_cast<unsigned>(i)
+               && ++spins < (1u << 20)) {
+        }
+        if (me == 1) put(static_cast<unsigned>(i));
+    }
+    ticks[me] = __builtin_amdgcn_s_memrealtime() - t0;  // 100 MHz
+}
+
+// Background load for the probe: streams a buffer until told to stop (or 2000 rounds).
+__global__ void handoff_probe_hog(const float4* buf, size_t n4, const volatile unsigned* stop, float* sink) {
+    float acc = 0.0f;
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    for (int it = 0; it < 2000 && *stop == 0u; it++)
+        for (int k = 0; k < 16; k++) {
+            const float4 v = buf[i];
+            acc += (v.x + v.y) + (v.z + v.w);
+            i += stride;
+            if (i >= n4) i -= n4;
+        }
+    if (acc == 1.2345f) *sink = acc;
+}
+
+using HandoffKernel = void (*)(unsigned*, int, int, unsigned long long*, unsigned*);
+static HandoffKernel handoff_kernel_for(int load_policy, bool device_store) {
+    switch (load_policy) {
+    case 0: return device_store ? handoff_probe_kernel<0, true> : handoff_probe_kernel<0, false>;
+    case 1: return device_store ? handoff_probe_kernel<kAuxNonTemporal, true> : handoff_probe_kernel<kAuxNonTemporal, false>;
+    case 2: return device_store ? handoff_probe_kernel<kAuxDeviceScope, true> : handoff_probe_kernel<kAuxDeviceScope, false>;
+    default: return nullptr;
+    }
+}
+
 }  // namespace gh
 
 // ====================================================================== C ABI
@@ -2468,6 +2522,63 @@ gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per
             if (r > 0) best = std::max(best, static_cast<double>(n4) * sizeof(float4) / (ms * 1e-3) / 1e9);
         }
         *gb_per_s = best;
+    });
+}
+
+gh_status gh_device_handoff_latency(int32_t load_policy, int32_t device_scope_store, int32_t peer, int32_t busy,
+                                    double* us_per_round_trip, int32_t* xcd_a, int32_t* xcd_b) {
+    return guard([&] {
+        require_gpu();
+        HandoffKernel kernel = handoff_kernel_for(load_policy, device_scope_store != 0);
+        if (!kernel || !us_per_round_trip || peer < 1 || peer > 15)
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "hand-off probe: load policy 0..2, peer workgroup 1..15"};
+        struct Scratch {  // released on every path out of this function
+            unsigned *cells = nullptr, *xcds = nullptr, *stop = nullptr;
+            unsigned long long* ticks = nullptr;
+            float4* big = nullptr;
+            float* sink = nullptr;
+            hipStream_t s1 = nullptr, s2 = nullptr;
+            ~Scratch() {
+                if (stop) *stop = 1u;
+                (void)hipDeviceSynchronize();
+                if (s1) (void)hipStreamDestroy(s1);
+                if (s2) (void)hipStreamDestroy(s2);
+                for (void* p : {static_cast<void*>(cells), static_cast<void*>(xcds), static_cast<void*>(ticks),
+                                static_cast<void*>(big), static_cast<void*>(sink)})
+                    if (p) (void)hipFree(p);
+                if (stop) (void)hipHostFree(stop);
+            }
+        } t;
+        const int rounds = 1000;
+        const size_t big_bytes = busy ? (size_t(2) << 30) : sizeof(float4);
+        dev_alloc(t.cells, 256);
+        dev_alloc(t.xcds, 16);
+        dev_alloc(t.ticks, 2);
+        HIP_CHECK(hipMalloc(&t.big, big_bytes));
+        HIP_CHECK(hipMemset(t.big, 0, big_bytes));
+        dev_alloc(t.sink, 1);
+        HIP_CHECK(hipHostMalloc(&t.stop, sizeof(unsigned), hipHostMallocCoherent));
+        *t.stop = 0u;
+        HIP_CHECK(hipStreamCreateWithFlags(&t.s1, hipStreamNonBlocking));
+        HIP_CHECK(hipStreamCreateWithFlags(&t.s2, hipStreamNonBlocking));
+        HIP_CHECK(hipDeviceSynchronize());
+        if (busy) {
+            hipLaunchKernelGGL(handoff_probe_hog, dim3(240), dim3(256), 0, t.s2, t.big, big_bytes / sizeof(float4),
+                               t.stop, t.sink);
+            HIP_CHECK(hipGetLastError());
+        }
+        hipLaunchKernelGGL(kernel, dim3(16), dim3(64), 0, t.s1, t.cells, peer, rounds, t.ticks, t.xcds);
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipStreamSynchronize(t.s1));
+        *t.stop = 1u;
+        HIP_CHECK(hipDeviceSynchronize());
+        unsigned long long ticks[2];
+        unsigned xcds[16];
+        HIP_CHECK(hipMemcpy(ticks, t.ticks, sizeof(ticks), hipMemcpyDeviceToHost));
+        HIP_CHECK(hipMemcpy(xcds, t.xcds, sizeof(xcds), hipMemcpyDeviceToHost));
+        *us_per_round_trip = static_cast<double>(ticks[0]) / 100.0 / rounds;
+        if (xcd_a) *xcd_a = static_cast<int32_t>(xcds[0]);
+        if (xcd_b) *xcd_b = static_cast<int32_t>(xcds[peer]);
     });
 }
 

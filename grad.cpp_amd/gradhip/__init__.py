@@ -109,6 +109,8 @@ SYMBOLS = {
     "gh_device_info": (C.c_int, [C.c_char_p, C.c_size_t, _i32p, _i32p]),
     "gh_device_read_bandwidth": (C.c_int, [C.c_size_t, C.c_int32, C.POINTER(C.c_double)]),
     "gh_device_reread_bandwidth": (C.c_int, [C.c_size_t, C.c_int32, C.POINTER(C.c_double)]),
+    "gh_device_handoff_latency": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double),
+                                            C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
 }
 
 _lib = None
@@ -159,6 +161,14 @@ def reread_bandwidth(nbytes: int, passes: int = 20) -> float:
     out = C.c_double(0.0)
     _check(load_library().gh_device_reread_bandwidth(nbytes, passes, C.byref(out)))
     return out.value
+
+
+def handoff_latency(load_policy: int, device_scope_store: bool, peer: int, busy: bool):
+    """(us per round trip, XCD of workgroup 0, XCD of workgroup `peer`) of a two-workgroup ping-pong."""
+    out, xa, xb = C.c_double(0.0), C.c_int32(-1), C.c_int32(-1)
+    _check(load_library().gh_device_handoff_latency(load_policy, 1 if device_scope_store else 0, peer,
+                                                    1 if busy else 0, C.byref(out), C.byref(xa), C.byref(xb)))
+    return out.value, xa.value, xb.value
 
 
 def pick_noalloc(logits_ptr: int, batch: int, vocab: int, history_ptr: int, history_stride: int, n_history: int,

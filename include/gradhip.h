@@ -348,6 +348,17 @@ gh_status gh_device_read_bandwidth(size_t bytes, int32_t repeats, double* gb_per
  * served from it; the rate over a range of sizes shows where that stops. */
 gh_status gh_device_reread_bandwidth(size_t bytes, int32_t passes, double* gb_per_s);
 
+/* Measurement aid with no counterpart in grad.cpp: what handing a word from one
+ * workgroup to another costs.  Workgroup 0 and workgroup `peer` (1..15; workgroups go
+ * round-robin over the XCDs, so 8 shares workgroup 0's XCD and 1 does not) bounce a
+ * counter 1000 times; *us_per_round_trip is the time per round trip (two hand-offs).
+ * load_policy: 0 ordinary, 1 non-temporal (served by the L2, never kept in the vector
+ * cache), 2 device scope.  device_scope_store: write-through store, or an ordinary
+ * one.  busy: 240 more workgroups stream from HBM meanwhile.  *xcd_a / *xcd_b (may be
+ * NULL) receive the XCDs the two workgroups ran on. */
+gh_status gh_device_handoff_latency(int32_t load_policy, int32_t device_scope_store, int32_t peer, int32_t busy,
+                                    double* us_per_round_trip, int32_t* xcd_a, int32_t* xcd_b);
+
 #ifdef __cplusplus
 }
 #endif
