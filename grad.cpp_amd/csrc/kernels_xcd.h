@@ -56,7 +56,7 @@ constexpr int kXcdRelayWave = 6;      // sums the partials of this workgroup's r
 constexpr int kXcdAttnWave = 7;       // attention of one slice (P2); takes no part in anything else
 constexpr int kXcds = 8, kWgPerXcd = 32;
 constexpr int kXcdUnit = 1024;        // bytes one streamer instruction moves
-constexpr int kXcdDepth = 16;         // loads a streamer keeps in flight
+constexpr int kXcdDepth = 12;         // loads a streamer keeps in flight
 constexpr int kAuxNonTemporal = 2;    // nt on gfx94x / gfx950 buffer instructions
 constexpr int kApCells = 66;          // cells of one attention partial: acc[64], m, l
 constexpr int kXcdMaxUnitsPerWg = 2 * kXcdTeamWaves;

@@ -30,7 +30,7 @@ def pytest_terminal_summary(terminalreporter):
     terminalreporter.write_line("logits rule, worst share of the allowance (max-norm, per-element):")
     named = {k: v for k, v in WORST.items() if k[:2] in ("c0", "c1", "c2", "c3", "c4")}
     for label in sorted(named):
-        a, b = named[label]
+        a, b = named[label][:2]
         terminalreporter.write_line(f"  {label}: {a:.3f} {b:.3f}")
     rest = {k: v for k, v in WORST.items() if k not in named}
     if rest:
@@ -38,3 +38,4 @@ def pytest_terminal_summary(terminalreporter):
         wb = max(rest, key=lambda k: rest[k][1])
         terminalreporter.write_line(f"  other comparisons ({len(rest)} labels): max-norm {rest[wa][0]:.3f} ({wa}), "
                                     f"per-element {rest[wb][1]:.3f} ({wb})")
+        terminalreporter.write_line(f"    that element: {rest[wb][2]}")

@@ -29,8 +29,8 @@ def rel_err(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
-# Worst observed values of the two logits rules per label, for the record a GPU
-# run prints at its end (tests/conftest.py).
+# Worst observed values of the two logits rules per label, and where the per-element
+# one was seen, for the record a GPU run prints at its end (tests/conftest.py).
 WORST = {}
 
 
@@ -50,10 +50,17 @@ def assert_logits_close(got, ref, tol=1e-4, what="", abs_term=None):
     a, b = np.asarray(got, np.float64), np.asarray(ref, np.float64)
     if abs_term is None:
         abs_term = 5e-6 * float(np.abs(b).max())
-    per = float((np.abs(a - b) / (tol * np.maximum(np.abs(a), np.abs(b)) + abs_term)).max())
+    share = np.abs(a - b) / (tol * np.maximum(np.abs(a), np.abs(b)) + abs_term)
+    per = float(share.max())
     label = what.split(" step ")[0].split(" decode ")[0] or "unnamed"
-    w = WORST.setdefault(label, [0.0, 0.0])
-    w[0], w[1] = max(w[0], e / tol), max(w[1], per)
+    w = WORST.setdefault(label, [0.0, 0.0, ""])
+    w[0] = max(w[0], e / tol)
+    if per > w[1]:
+        i = int(share.reshape(-1).argmax())
+        big = max(float(np.abs(b).max()), 1e-30)
+        w[1] = per
+        w[2] = (f"{what or 'unnamed'}, element {i}: |ref| = {abs(b.reshape(-1)[i]) / big:.4f} of the step's largest, "
+                f"|d| = {abs(a.reshape(-1)[i] - b.reshape(-1)[i]) / big:.2e} of it")
     assert e <= tol, f"{what}: max|d|/max|ref| = {e:.3e} > {tol}"
     assert per <= 1.0, f"{what}: per-element rule exceeded ({per:.3f} of the allowance)"
 

@@ -30,6 +30,21 @@ def models():
 
 @pytest.mark.parametrize("name", sorted(SHAPES))
 def test_auto_engine_is_persistent_and_steps_match(models, name):
+    """Every step of a full context against the checker.
+
+    `llama-d768` comes closest to the per-element rule of `assert_logits_close`
+    (0.75 to 0.80 of the allowance; the max-norm rule stays at 0.05 of its own).  The
+    elements that get there are logits near zero: |ref| between 0.0006 and 0.017 of the
+    step's largest logit (4.2 to 4.9 with these std-0.05 weights), off by 3.6e-6 to
+    5.0e-6 of that largest logit, where the rule's absolute term allows 5e-6.  It is not
+    the summation order of one kernel: the all-to-all kernel, the XCD kernel and the
+    graph engine, which sum in three different orders, land on the same elements
+    (step 21 element 831, step 69 element 609, step 6 element 845, step 90, step 85)
+    with the same sign and the same size to 3 % (the engines are held to each other five
+    times as tightly as to the checker, the 2e-5 comparison below).  What they share is the
+    GPU's arithmetic against the checker's: fused multiply-adds and the hardware's
+    exp and reciprocal square root against unfused AVX2 sums and libm.  The run's closing
+    record names the element and both ratios."""
     cfg, W, om, gm = models[name]
     auto = G.Session(gm)  # picks the persistent engine for these shapes
     forced = G.Session(gm, engine=G.ENGINE_PERSISTENT, shuffle_pages=True, page_tokens=8)
