@@ -193,7 +193,7 @@ def cpu_baseline(synth, W2):
             "single_thread": out["c2"]["threads_1"]["decode_tok_s"], "host_cpus": ncpu, "configs": out}
 
 
-def phase_stamps(xcd=False):
+def phase_stamps(xcd=False, greedy=False, row_picks=False):
     """Mean phase durations of one token of c2 on a persistent kernel, from the stamps
     workgroup 0 leaves (GRADHIP_PROF_DUMP).  The all-to-all kernel: per step one stamp
     after the pick, five per layer, one when the logits rows have arrived, one at the
@@ -207,9 +207,11 @@ def phase_stamps(xcd=False):
     cfg = synth.PRESETS["c2"]
     gm = G.Model.from_tensors(cfg, synth.make_weights(cfg, 1002))
     gs = G.Session(gm, engine=G.ENGINE_PERSISTENT,
-                   flags=G.FLAG_XCD_PERSISTENT if xcd else G.FLAG_CLASSIC_PERSISTENT)
+                   flags=(G.FLAG_XCD_PERSISTENT if xcd else G.FLAG_CLASSIC_PERSISTENT)
+                   | (G.FLAG_ROW_PICKS if row_picks else 0))
     gs.prefill(synth.uniform_tokens(32, cfg.vocab, 2002)[None, :])
-    gs.decode(224, G.sampling(0.8, 40, 0.9, 1.1), seed=2002)
+    gs.decode(224, G.sampling(greedy=True, repetition_penalty=1.0) if greedy else G.sampling(0.8, 40, 0.9, 1.1),
+              seed=2002)
     gpu_us = gs.last_timing()["decode_ms"] * 1e3 / 224
     gs.close()  # writes the dump: stamps, "0", three clock readings per pick, "0", counters
     words = open(dump).read().split()
@@ -226,7 +228,8 @@ def phase_stamps(xcd=False):
     pk = np.array([int(x) for x in words[z + 1:z2]], dtype=np.float64) / 100.0
     pk = pk[: len(pk) // 3 * 3].reshape(-1, 3)[3:]
     out = {
-        "workload": "c2, one launch of 224 pick + step rounds, contexts 33..256", "steps_averaged": int(k),
+        "workload": "c2%s, one launch of 224 pick + step rounds, contexts 33..256" % (" with greedy picks" if greedy else ""),
+        "steps_averaged": int(k),
         "kernel": "xcd_decode_kernel" if xcd else "persist_decode_kernel",
         "us_per_token_events": round(gpu_us, 2), "us_per_token_stamps": round(float(m.sum()), 2),
         "pick_until_token_seen": round(float(m[0]), 2),
@@ -281,6 +284,11 @@ def main():
                     help="only run one 224-step launch of the batch-1 workload with the persistent kernel's "
                          "in-kernel phase stamps on (workgroup 0's clock at the end of every phase) and "
                          "print the mean duration of every phase of a token")
+    ap.add_argument("--row-picks", action="store_true",
+                    help="batch-1 legs and --phase-stamps: every pick by one workgroup from the whole row of "
+                         "logits (GH_FLAG_ROW_PICKS) instead of by every workgroup from candidates")
+    ap.add_argument("--greedy-picks", action="store_true",
+                    help="with --phase-stamps: greedy picks without a penalty instead of the workload's sampler")
     ap.add_argument("--kernel", default="auto", choices=["auto", "classic", "xcd"],
                     help="pin the batch-1 legs to one of the persistent engine's two kernels (the all-to-all "
                          "kernel or the XCD-sharded one); auto: by position, as sessions do by default")
@@ -296,7 +304,7 @@ def main():
                     help="the same for the XCD-sharded persistent kernel (eight stamps per layer)")
     a = ap.parse_args()
     if a.phase_stamps or a.phase_stamps_xcd:
-        phase_stamps(xcd=a.phase_stamps_xcd)
+        phase_stamps(xcd=a.phase_stamps_xcd, greedy=a.greedy_picks, row_picks=a.row_picks)
         return
     if a.handoff_probe:
         import gradhip as G
@@ -353,6 +361,8 @@ def main():
     sample = G.sampling(*opts)
 
     b1_flags = {"auto": 0, "classic": G.FLAG_CLASSIC_PERSISTENT, "xcd": G.FLAG_XCD_PERSISTENT}[a.kernel]
+    if a.row_picks:
+        b1_flags |= G.FLAG_ROW_PICKS
     if a.step_loop:
         gs = G.Session(gm, engine=engine, flags=b1_flags)
         prompt = synth.uniform_tokens(32, cfg.vocab, 2002)
@@ -458,13 +468,13 @@ def main():
         cfg0 = synth.PRESETS["c0"]
         gm0 = G.Model.from_tensors(cfg0, synth.make_weights(cfg0, 1000))
         r0 = run_decode(G, synth, gm0, cfg0, 1, 16, 80, 80, G.sampling(greedy=True, repetition_penalty=1.2),
-                        2000, engine)
+                        2000, engine, b1_flags & G.FLAG_ROW_PICKS)
         line["c0"] = leg("c0: GPT-2 block 'small' (d512 L6 H8 F2048 V5000 C96), batch 1, 16-token prompt, "
                          "80 greedy steps, repetition penalty 1.2 (the reference's default)", r0, 1)
         del gm0
         cfg1 = synth.PRESETS["c1"]
         gm1 = G.Model.from_tensors(cfg1, synth.make_weights(cfg1, 1001))
-        r1m = run_decode(G, synth, gm1, cfg1, 1, 32, 224, 224, greedy, 2001, engine)
+        r1m = run_decode(G, synth, gm1, cfg1, 1, 32, 224, 224, greedy, 2001, engine, b1_flags & G.FLAG_ROW_PICKS)
         line["c1"] = leg("c1: GPT-2 block 'medium' (d768 L8 H12 F3072 V16000 C256), batch 1, 32-token prompt, "
                          "224 greedy steps", r1m, 1)
         del gm1

@@ -381,6 +381,7 @@ struct Session {
     bool xcd = false;         // the kernel and its buffers are ready
     bool xcd_always = false;  // GH_FLAG_XCD_PERSISTENT: every launch takes it
     bool xcd_row_lds = false;
+    bool row_picks_only = false;  // GH_FLAG_ROW_PICKS
     Cell* xcells = nullptr;
     unsigned xcd_cells_count = 0;
     unsigned xcd_launches = 0;
@@ -402,6 +403,16 @@ struct Session {
     gh_timing timing{};
 
     ~Session() {
+#ifdef GH_PICK_TICKS
+        {
+            unsigned long long t[32] = {};
+            if (hipMemcpyFromSymbol(t, HIP_SYMBOL(g_pick_ticks), sizeof(t)) == hipSuccess) {
+                std::fprintf(stderr, "pick ticks (10 ns, summed):");
+                for (unsigned long long v : t) std::fprintf(stderr, " %llu", v);
+                std::fprintf(stderr, "\n");
+            }
+        }
+#endif
         if (prof) {
             // Developer aid: phase-end timestamps of the last persistent launch.
             std::vector<unsigned long long> host(prof_cap);
@@ -935,6 +946,7 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     p.n_picks = n_picks;
     p.start_with_pick = start_with_pick ? 1 : 0;
     p.tok0 = tok0;
+    p.wg_picks = s.row_picks_only ? 0 : 1;
     p.epoch = s.epoch;
     p.arrive_base = s.arrive_total;
     p.spin_limit = 1u << 18;
@@ -1149,6 +1161,7 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     HIP_CHECK(hipDeviceGetAttribute(&lds_bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
     const size_t reserve = 8192;
     s.pick_global_scratch = (o.flags & GH_FLAG_PICK_GLOBAL_SCRATCH) != 0;
+    s.row_picks_only = (o.flags & GH_FLAG_ROW_PICKS) != 0;
     s.use_prompt_pass = (o.flags & GH_FLAG_STEPWISE_PROMPT) == 0;
     s.pick_row_in_lds = !s.pick_global_scratch
                         && (V + kPickWorkFloats) * sizeof(float) + reserve <= static_cast<size_t>(lds_bytes);
@@ -1169,7 +1182,10 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
             const size_t pick = (s.pick_row_in_lds ? V : 0) + kPickWorkFloats;
             s.persist_lds = std::max(work, pick) * sizeof(float);
             s.persist_grid = std::min(prop.multiProcessorCount, 256);
-            s.cells_count = 6 * d + F + 1;
+            // the exchange cells, the token cell (and one of padding), then what the workgroups
+            // leave for a pick each of them makes itself: nine planes of one cell per
+            // workgroup and a stop word
+            s.cells_count = 6 * d + F + 2 + 9 * static_cast<size_t>(s.persist_grid) + 1;
             dev_alloc(s.cells, s.cells_count);
             // Rows of the cache written earlier in a launch by other workgroups are read
             // with ordinary loads.  That is sound only because a row is never read before
@@ -2469,6 +2485,12 @@ gh_status gh_session_last_timing(const gh_session* s, gh_timing* out) {
     return guard([&] {
         if (!s || !out) throw ApiError{GH_ERR_INVALID_ARGUMENT, "null argument"};
         *out = s->impl->timing;
+        out->row_picks = 0;
+        if (s->impl->ctl) {
+            unsigned n = 0;
+            HIP_CHECK(hipMemcpy(&n, &s->impl->ctl->row_picks, sizeof(n), hipMemcpyDeviceToHost));
+            out->row_picks = static_cast<int32_t>(n);
+        }
     });
 }
 

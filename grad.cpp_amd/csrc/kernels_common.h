@@ -88,6 +88,29 @@ __device__ __forceinline__ float wave_max(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// The largest value of a wavefront and, among equal ones, the lowest index that came
+// with it: the same six steps on a (value, index) pair.  Every lane returns the result.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void first_max_step(float& v, int& i) {
+    const float ov = dpp_move<CTRL, ROW_MASK>(v, v);
+    const int oi = __builtin_amdgcn_update_dpp(i, i, CTRL, ROW_MASK, 0xF, false);
+    if (ov > v || (ov == v && oi < i)) {
+        v = ov;
+        i = oi;
+    }
+}
+
+__device__ __forceinline__ void wave_first_max(float& v, int& i) {
+    first_max_step<0xB1, 0xF>(v, i);
+    first_max_step<0x4E, 0xF>(v, i);
+    first_max_step<0x141, 0xF>(v, i);
+    first_max_step<0x140, 0xF>(v, i);
+    first_max_step<0x142, 0xA>(v, i);
+    first_max_step<0x143, 0xC>(v, i);
+    v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+    i = __builtin_amdgcn_readlane(i, 63);
+}
+
 // Running total over the lanes of a wavefront, this lane's own value included:
 // shifts inside each row of 16, then the totals of the rows before.
 template <int CTRL, int ROW_MASK>

@@ -71,7 +71,8 @@ __device__ __forceinline__ LayerPtrs layer_at(const float* layer0, int l) {
 struct PersistCtl {
     unsigned abort;     // set by any workgroup that gave up waiting
     unsigned where;     // phase tag it was waiting for (diagnostics)
-    unsigned pad[30];
+    unsigned row_picks;  // picks workgroup 0 made from the whole row (the others: every workgroup, from candidates)
+    unsigned pad[29];
     unsigned arrive[16 * 32];  // logits-complete counters, one per 128-byte line
     unsigned xcd_count[8 * 32];  // workgroups that have started on each XCD, one counter per line (kernels_xcd.h)
 };
@@ -85,7 +86,10 @@ struct PersistParams {
     KvLayout kv;
     // One block of exchange cells, in this order: x after a layer [d], x after the
     // attention half [d], q [d], new key [d], new value [d], attention output [d],
-    // FFN hidden [F], the picked token [1].  The kernel addresses them from the one
+    // FFN hidden [F], the picked token [1] (+ 1 unused), then what the workgroups leave for
+    // a pick that each of them makes itself: planes of one cell per workgroup (greedy:
+    // largest logit, its index; top-k: four values, four indices, the fifth value) and
+    // the host's stop request as workgroup 0 read it [1].  The kernel addresses them from the one
     // base: eight pointers held through the whole token loop are sixteen scalar
     // registers that would otherwise be parked in vector lanes and fetched back.
     Cell* cells;
@@ -99,6 +103,7 @@ struct PersistParams {
     int n_picks;       // picks in this launch
     int start_with_pick;  // the first pick uses the logits already in memory
     int tok0;             // >= 0: the token of step 0 (not yet in the history: the kernel records it)
+    int wg_picks;         // picks that follow a step may be made by every workgroup from candidates
     unsigned epoch;    // tag base of this launch; (epoch + s) never repeats in a session
     unsigned arrive_base;  // logits phases completed before this launch
     PickParams pick;
@@ -267,6 +272,7 @@ __device__ __forceinline__ bool persist_pick(const PersistParams& p, float* lds,
         __hip_atomic_store(&p.hist[pk.n_hist], chosen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         cell_put(tok_cell, __int_as_float(chosen), tok_tag);
         if constexpr (FEED) feed_put(p, i_pick, chosen);
+        __hip_atomic_fetch_add(&p.ctl->row_picks, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (pp) pp[1] = __builtin_amdgcn_s_memrealtime();
     }
     return true;
@@ -402,6 +408,14 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     unsigned arrive_gen = p.arrive_base;
     int n_stamp = 0;
     bool ended = false;  // a picked token was the stop token
+    // Greedy picks of this launch are made by every workgroup from per-workgroup maxima
+    // (the pick that opens a launch on logits of an earlier one is workgroup 0's).
+    const bool fast_greedy = p.wg_picks != 0 && p.pick.greedy != 0;
+    // Top-k picks likewise, when a workgroup's rows are one item per wavefront (64 values)
+    // and every workgroup has an item (at least eight values).
+    const bool fast_topk = p.wg_picks != 0 && p.pick.greedy == 0 && p.pick.top_k > 0 && p.pick.top_k <= 64 && p.pick.top_k < V
+                           && (V + RL - 1) / RL <= G * kPersistWaves && V >= G * RL;
+    bool pairs_out = false;  // the last logits phase left the planes for the pick that follows
     auto stamp = [&]() {
         if (p.prof && wg == 0 && tid == 0 && n_stamp < p.prof_cap) p.prof[n_stamp] = __builtin_amdgcn_s_memrealtime();
         n_stamp++;
@@ -426,7 +440,94 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         // ===== pick before step s (text_gen.cpp:48-61): the first one of a launch may
         // use logits that are already in memory, later ones follow step s - 1.  One call
         // site: the sampler is the largest piece of code in the kernel.
-        if ((!FEED || !ended) && i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick)) {
+        const bool pick_here =
+            (!FEED || !ended) && i_pick < p.n_picks && s >= p.n_prompt && (s > 0 || p.start_with_pick);
+        // Layer 0's QKV operands are fetched while the token is on its way.
+        QkvOperands<KD, PRO> qo;
+        auto load_qo0 = [&]() {
+            const LayerPtrs w0l = layer_at<KD, KF, MODERN>(p.layer0, 0);
+            if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, w0l, first, p.pos0 + s, lane, qo);
+            else qo = QkvOperands<KD, PRO>{};  // nothing to keep alive across steps
+        };
+        int tok_fast = 0;
+        bool tok_known = false;
+        if (pick_here && pairs_out) {
+            // ===== a pick without a picker (text_gen.cpp:48-61, :135-209).  The logits phase
+            // of step s - 1 left, per workgroup, its largest penalised logit and first index
+            // (greedy), or its four largest scaled ones and the fifth's value (top-k of at most
+            // 64).  Every workgroup reads all of them and makes the same pick itself: the
+            // token needs one exchange and no row is read back.
+            asm volatile("" : "+v"(tid));
+            wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+            lane = tid & 63;
+            first = wg + G * wave;
+            unsigned long long* pp =
+                (p.prof && wg == 0 && tid == 0 && i_pick < 1024) ? p.prof + p.prof_cap / 2 + 4 * i_pick : nullptr;
+            if (pp) pp[2] = __builtin_amdgcn_s_memrealtime();
+            if (s < p.n_steps) load_qo0();
+            const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
+                                 + static_cast<unsigned>(L)) * 8u + 7u;
+            const Cell* pc = p.cells + 6 * D + F + 2;
+            float* g = lds;  // the gathered planes; xs and vin hold nothing between steps
+            bool stop = false;
+            if (fast_greedy) {
+                if (!gather_cells(pc, 2 * G + 1, tt, g, p)) return;
+                if (pp) pp[0] = __builtin_amdgcn_s_memrealtime();
+                float best = -INFINITY;
+                int bi = 0x7FFFFFFF;
+                for (int j = lane; j < G; j += 64) {
+                    const float v = g[j];
+                    const int i = __float_as_int(g[G + j]);
+                    if (v > best || (v == best && i < bi)) {
+                        best = v;
+                        bi = i;
+                    }
+                }
+                wave_first_max(best, bi);
+                tok_fast = bi == 0x7FFFFFFF ? 0 : bi;
+                stop = FEED && __float_as_int(g[2 * G]) != 0;
+                tok_known = true;
+            } else {
+                PickParams pk = p.pick;
+                pk.pick_idx = p.pick.pick_idx + i_pick;
+                const float u = pick_draw(pk, 0);  // needs no logits
+                PTICK_BEGIN();
+                if (!gather_cells(pc, 9 * G + 1, tt, g, p)) return;
+                PTICK(9);
+                if (pp) pp[0] = __builtin_amdgcn_s_memrealtime();
+                // The four planes hold every value that can survive the cut when the largest
+                // value a workgroup kept back is below the k-th largest of the planes; the
+                // sampler checks that and declines otherwise (workgroup 0 then picks from the row).
+                float kept_back = -INFINITY;
+                for (int j = lane; j < G; j += 64) kept_back = fmaxf(kept_back, g[8 * G + j]);
+                kept_back = wave_max(kept_back);
+                PTICK(10);
+                float* red = g + 9 * G + 8;
+                int* ishare = reinterpret_cast<int*>(red + 8);
+                float* work = g + 9 * G + 64;
+                const int c = sample_topk_fast<kPersistThreads, 2>(g, 4 * G, 1.0f, pk.top_k, pk.top_p, u, work, red, ishare,
+                                                                   reinterpret_cast<const int*>(g + 4 * G), kept_back, V - 1);
+                stop = FEED && __float_as_int(g[9 * G]) != 0;
+                __syncthreads();
+                tok_fast = c;
+                tok_known = c >= 0 || stop;
+#ifdef GH_PICK_TICKS
+                if (wg == 0 && tid == 0) g_pick_ticks[c >= 0 ? 12 : 13] += 1;
+#endif
+            }
+            if (stop) tok_fast = -1;  // the host asked for the run to end here
+            if (tok_known) {
+                if (wg == 0 && tid == 0) {
+                    if (tok_fast >= 0)
+                        __hip_atomic_store(&p.hist[p.pick.n_hist + i_pick], tok_fast, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                    if constexpr (FEED) feed_put(p, i_pick, tok_fast);
+                }
+                if (pp) pp[1] = __builtin_amdgcn_s_memrealtime();
+                i_pick++;
+            }
+        }
+        if (pick_here && !tok_known) {
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
                                  + static_cast<unsigned>(L)) * 8u + (s == 0 ? 6u : 7u);
             if (!persist_pick<ROW_LDS, FEED>(p, lds, i_pick, arrive_gen, tt, s > 0, G, p.cells + 6 * p.d + p.F)) return;
@@ -438,8 +539,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 __syncthreads();
             }
         }
+        pairs_out = false;
         stamp();
         if ((FEED && ended) || s >= p.n_steps) break;
+        if (FEED && tok_known && tok_fast < 0) return;
         asm volatile("" : "+v"(tid));  // as in the layer loop below
         wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         lane = tid & 63;
@@ -451,13 +554,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
         };
         const bool want_logits = (s >= p.n_prompt - 1) || p.logit_log != nullptr || s == p.n_steps - 1;
 
-        // Operands of layer 0's QKV are fetched while the token arrives.
-        QkvOperands<KD, PRO> qo;
-        {
-            const LayerPtrs w0l = layer_at<KD, KF, MODERN>(p.layer0, 0);
-            if (has_qkv) load_qkv_operands<KD, PRO, MODERN>(p, w0l, first, pos, lane, qo);
-            else qo = QkvOperands<KD, PRO>{};  // nothing to keep alive across steps
-        }
+        if (!tok_known) load_qo0();
 
         // ---- token and embedding (inference.cpp:159-182)
         int tok;
@@ -470,6 +567,9 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             } else {
                 tok = p.hist[pos];
             }
+        } else if (tok_known) {
+            tok = tok_fast;
+            if constexpr (FEED) ended = tok == p.stop_token;  // this step is the last one
         } else {
             // the pick that followed step s-1 (or opened the launch)
             const unsigned tt = ((p.epoch + static_cast<unsigned>(s)) * static_cast<unsigned>(L + 1)
@@ -904,6 +1004,34 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             // store (a conditional fetch makes the compiler spill the rows to scratch)
 #pragma unroll
             for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(first * RL + r, V - 1), D, lane, wr[r]);
+            // A pick every workgroup makes itself follows: beside the rows go this workgroup's
+            // largest penalised logit and its first index (greedy) or its four largest
+            // penalised, scaled logits with their indices and the value of the fifth (top-k).
+            // logits_with_penalty (text_gen.cpp:14-33) counts once per occurrence in the last
+            // 50 tokens, which every wavefront holds a lane each.
+            const bool pick_next = (!FEED || !ended) && i_pick < p.n_picks && s + 1 >= p.n_prompt;
+            const bool publish = (fast_greedy || fast_topk) && pick_next;
+            int window = 0;
+            int* win = reinterpret_cast<int*>(ascr) + 2 * kPersistWaves;  // [64] the window's tokens, in LDS
+            float* mine8 = ascr + 2 * kPersistWaves + 64;                 // [64] the workgroup's values (top-k)
+            unsigned stop_word = 0u;
+            if (publish) {
+                if (p.pick.penalty != 1.0f) {
+                    const int n_hist = p.pick.n_hist + i_pick;
+                    window = min(kPenaltyWindow, n_hist);
+                    if (tid < window)
+                        win[tid] = __hip_atomic_load(&p.hist[n_hist - window + tid], __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if constexpr (FEED) {
+                    // the host's stop request: one trip over the bus behind the rows of E
+                    if (wg == 0 && tid == 0)
+                        stop_word = __hip_atomic_load(p.stop_request, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+            }
+            const float inv_t = 1.0f / p.pick.temperature;
+            float best = -INFINITY;
+            int best_row = 0x7FFFFFFF;
             __syncthreads();
             if (!gather_cells(p.cells, D, tag_of(L - 1, 4), xs, p)) return;
             stamp();
@@ -913,6 +1041,27 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 float out[RL];
 #pragma unroll
                 for (int r = 0; r < RL; r++) out[r] = dot_row<KD>(rows[r], h);
+                if (publish) {
+                    const int win_tok = lane < window ? win[lane] : -1;
+#pragma unroll
+                    for (int r = 0; r < RL; r++) {
+                        const int row = item * RL + r;
+                        float v = out[r];
+                        if (window > 0) {
+                            const int times = __popcll(__ballot(win_tok == row));
+                            for (int c = 0; c < times; c++) v = (v > 0.0f) ? v / p.pick.penalty : v * p.pick.penalty;
+                        }
+                        if (fast_greedy) {
+                            if (row < V && v > best) {  // rows ascend: the first maximum stays
+                                best = v;
+                                best_row = row;
+                            }
+                        } else if (lane == 0) {
+                            v *= inv_t;  // text_gen.cpp:140-143
+                            mine8[wave * RL + r] = (row < V && v == v) ? v : -INFINITY;
+                        }
+                    }
+                }
                 if (lane == 0) {
 #pragma unroll
                     for (int r = 0; r < RL; r++) {
@@ -933,9 +1082,67 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                 for (int r = 0; r < RL; r++) load_row<KD>(p.E, min(item * RL + r, V - 1), D, lane, wl[r]);
                 emit(item, wl);
             }
-            // this workgroup's rows are out: signal
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
+            PTICK_BEGIN();
+            if (publish) {
+                const unsigned tt = ((p.epoch + static_cast<unsigned>(s + 1)) * static_cast<unsigned>(L + 1)
+                                     + static_cast<unsigned>(L)) * 8u + 7u;
+                Cell* pc = p.cells + 6 * D + F + 2;
+                if (fast_greedy) {
+                    if (lane == 0) {
+                        ascr[wave] = best;
+                        ascr[kPersistWaves + wave] = __int_as_float(best_row);
+                    }
+                    __syncthreads();
+                    if (wave == 0) {
+                        best = lane < kPersistWaves ? ascr[lane] : -INFINITY;
+                        best_row = lane < kPersistWaves ? __float_as_int(ascr[kPersistWaves + lane]) : 0x7FFFFFFF;
+                        first_max_step<0xB1, 0xF>(best, best_row);
+                        first_max_step<0x4E, 0xF>(best, best_row);
+                        first_max_step<0x141, 0xF>(best, best_row);  // lanes 0..7 hold the workgroup's pair
+                    }
+                    if (tid == 0) {
+                        cell_put(pc + wg, best, tt);
+                        cell_put(pc + G + wg, __int_as_float(best_row), tt);
+                        if (wg == 0) cell_put(pc + 2 * G, __int_as_float(stop_word != 0u ? 1 : 0), tt);
+                    }
+                } else {
+                    // Values [4 G], indices [4 G], the fifth value [G], the stop word.  A
+                    // workgroup's j-th largest sits at (j / 2) * 2 G + 2 wg + j % 2: read as a row
+                    // of 4 G by 2 G threads, two elements each, every second thread of every
+                    // wavefront then holds a workgroup's maximum, which is what keeps the
+                    // sampler's first threshold close to the k-th largest.  Wavefront 0 takes
+                    // the largest five times (equal values: the lower row, which is the lower lane).
+                    __syncthreads();
+                    if (wave == 0) {
+                        float rest = mine8[lane];
+                        const int row = (wg + G * (lane >> 3)) * RL + (lane & 7);
+#pragma unroll
+                        for (int j = 0; j < 5; j++) {
+                            const float sel = wave_max(rest);
+                            const unsigned long long at = __ballot(rest == sel);
+                            if (lane == __ffsll(static_cast<long long>(at)) - 1) {
+                                if (j < 4) {
+                                    Cell* c = pc + (j >> 1) * 2 * G + 2 * wg + (j & 1);
+                                    cell_put(c, sel, tt);
+                                    cell_put(c + 4 * G, __int_as_float(row), tt);
+                                } else {
+                                    cell_put(pc + 8 * G + wg, sel, tt);
+                                }
+                                rest = -INFINITY;
+                            }
+                        }
+                        if (wg == 0 && lane == 0) cell_put(pc + 9 * G, __int_as_float(stop_word != 0u ? 1 : 0), tt);
+                    }
+                }
+                pairs_out = true;
+                PTICK(8);
+            }
+            // This workgroup's rows are out: signal.  The count follows the rows for the
+            // picker that reads them back; in a launch of greedy picks nobody does.
+            if (!fast_greedy) {
+                __builtin_amdgcn_s_waitcnt(0);
+                __syncthreads();
+            }
             arrive_gen++;
             if (tid == 0)
                 __hip_atomic_fetch_add(&p.ctl->arrive[(wg & 15) * 32], 1u, __ATOMIC_RELAXED,

@@ -352,37 +352,40 @@ __device__ __forceinline__ float wave_total_in_order(float x, int n) {
     return acc;
 }
 
-// The same two walks over a list that sits in LDS (n a multiple of 8, the list
-// padded with zeros): every lane reads every element (one address per read, a
-// broadcast) and runs the chain of additions itself.  Same order of additions,
-// same results; no lane-to-scalar move in front of each one.
-__device__ __forceinline__ float lds_total_in_order(const float* x, int n) {
-    float acc = 0.0f;
-    for (int j = 0; j < n; j += 8) {
-        float v[8];
+// Running sums in the order a serial loop forms them, p[l] = ((x[0] + x[1]) + ...) + x[l],
+// for the first n lanes (n a multiple of 8, x >= 0 and 0 from lane n on), in n steps of
+// one shifted addition each: after step t lane l holds x[l - t] + ... + x[l] added left to
+// right, and once t reaches l that is the whole prefix and stays it (what shifts into
+// lane 0 is a zero, and 0 + x[0] is x[0]).  No trip to LDS and no lane-to-scalar move.
+__device__ __forceinline__ float wave_serial_prefix(float x, int n) {
+    float acc = x;
+    for (int t = 0; t < n; t += 8) {
 #pragma unroll
-        for (int q = 0; q < 8; q++) v[q] = x[j + q];
-#pragma unroll
-        for (int q = 0; q < 8; q++) acc += v[q];
+        for (int q = 0; q < 8; q++)
+            acc = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc), 0x138 /* wave_shr:1 */, 0xF, 0xF,
+                                                             true))
+                  + x;
     }
     return acc;
 }
 
-__device__ __forceinline__ int lds_prefixes_below(const float* x, int n, float thr) {
-    float acc = 0.0f;
-    int below = 0;
-    for (int j = 0; j < n; j += 8) {
-        float v[8];
-#pragma unroll
-        for (int q = 0; q < 8; q++) v[q] = x[j + q];
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            acc += v[q];
-            below += (acc < thr) ? 1 : 0;
-        }
-    }
-    return below;
-}
+// Developer aid (-DGH_PICK_TICKS): time thread 0 of workgroup 0 spends in each stage of
+// the fast sampler, summed over picks, on the 100 MHz clock.
+#ifdef GH_PICK_TICKS
+__device__ unsigned long long g_pick_ticks[32];
+#define PTICK_BEGIN() unsigned long long ptick_last_ = __builtin_amdgcn_s_memrealtime()
+#define PTICK(i)                                                             \
+    do {                                                                     \
+        if (threadIdx.x == 0 && blockIdx.x == 0) {                           \
+            const unsigned long long t_ = __builtin_amdgcn_s_memrealtime();  \
+            g_pick_ticks[i] += t_ - ptick_last_;                             \
+            ptick_last_ = t_;                                                \
+        }                                                                    \
+    } while (0)
+#else
+#define PTICK_BEGIN() do {} while (0)
+#define PTICK(i) do {} while (0)
+#endif
 
 constexpr int kFastCandCap = 512;
 // LDS floats the fast sampler needs: candidate values, indices and ranks, the
@@ -405,9 +408,15 @@ constexpr int kFastLdsFloats = 3 * kFastCandCap + 3 * 64 + 128;
 // NT = threads of the workgroup and ROUNDS = elements per thread (compile time,
 // so that a thread's elements sit at immediate offsets and stay in registers
 // between the two passes); needs V <= ROUNDS * NT.
+// ids: the token id of every element when val is not a row of logits but a list of
+// candidates from one (index order means token order); outside: the largest value
+// that is not in val, below which the k-th largest must not fall for the cut to be
+// the row's (-1 otherwise); last_id: the row's last token id (the walk's answer when
+// rounding keeps the running sum below the draw, text_gen.cpp:202-208).
 template <int NT, int ROUNDS>
 __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int k, float top_p, float u,
-                                       float* work, float* red, int* ishare) {
+                                       float* work, float* red, int* ishare, const int* ids = nullptr,
+                                       float outside = -INFINITY, int last_id = 0) {
     constexpr int nt = NT, nw = NT / 64;
     static_assert(ROUNDS <= 64, "one mask bit per element of a thread");
     static_assert(NT >= kFastCandCap, "every candidate needs a thread");
@@ -419,6 +428,7 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
     asm volatile("" : "+v"(tid), "+s"(V));
     const int lane = tid & 63, wave = tid >> 6;
     if (V > ROUNDS * NT) return -1;
+    PTICK_BEGIN();
     float* cand_v = work;
     int* cand_i = reinterpret_cast<int*>(work + kFastCandCap);
     int* rank = cand_i + kFastCandCap;
@@ -452,6 +462,7 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         ridx[tid] = 0;
     }
     __syncthreads();
+    PTICK(0);
     float T = red[0];
     for (int w = 1; w < nw; w++) T = fminf(T, red[w]);
 
@@ -477,13 +488,17 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
             if (slot < kFastCandCap) {
                 const int i = r * nt + tid;
                 cand_v[slot] = val[i] * inv_t;
-                cand_i[slot] = i;
+                cand_i[slot] = ids ? ids[i] : i;
             }
             slot++;
         }
     }
     __syncthreads();
+    PTICK(1);
     const int c = ishare[1];
+#ifdef GH_PICK_TICKS
+    if (threadIdx.x == 0 && blockIdx.x == 0) g_pick_ticks[14] += c;
+#endif
     if (c > kFastCandCap || c < k) return -1;  // uniform: every thread reads the same count
 
     // descending rank of every candidate (ties: lower slot first), all threads:
@@ -504,6 +519,7 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         if (L < c && partial) atomicAdd(&rank[L], partial);
     }
     __syncthreads();
+    PTICK(2);
     if (tid < c) {
         const int r = rank[tid];
         if (r < 64) {
@@ -512,10 +528,15 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         }
     }
     __syncthreads();
+    PTICK(3);
     // the cut keeps ties at the threshold (text_gen.cpp:150-154)
     const float thr = sv[k - 1];
+    if (!(outside < thr)) return -1;  // uniform
     const unsigned long long kept = __ballot(sv[lane] >= thr);
     const int S = __popcll(kept);
+#ifdef GH_PICK_TICKS
+    if (threadIdx.x == 0 && blockIdx.x == 0) g_pick_ticks[15] += S;
+#endif
     if (S == 64 && c > 64) return -1;  // the ties may run past what one wavefront holds
     {
         // position of every survivor in index order
@@ -527,6 +548,7 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         if (lane < S && partial) atomicAdd(&ridx[lane], partial);
     }
     __syncthreads();
+    PTICK(4);
     if (tid < 64) {
         const int n = min(64, (S + 7) & ~7);
         const bool live = lane < S;
@@ -534,7 +556,6 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         const int ri = live ? ridx[lane] : lane;
         const float e = live ? expf(v - sv[0]) : 0.0f;
         float* in_order = reinterpret_cast<float*>(perm);  // [64] a value per survivor, index order
-        float* walk = cand_v;                               // [64] the list an ordered walk goes over
         // index-order copies of e and of the token ids
         perm[lane] = 0;
         perm[64 + lane] = 0x7FFFFFFF;
@@ -545,38 +566,37 @@ __device__ inline int sample_topk_fast(const float* val, int V, float inv_t, int
         }
         __builtin_amdgcn_wave_barrier();
         const float eo = in_order[lane];
-        const float inv_sum = 1.0f / lds_total_in_order(in_order, n);
+        const float inv_sum =
+            1.0f / __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_serial_prefix(eo, n)), n - 1));
         float po = eo * inv_sum;  // index order
         if (top_p < 1.0f) {
             float pr = e * inv_sum;  // descending order
-            walk[lane] = pr;
-            __builtin_amdgcn_wave_barrier();
             // first position whose running sum reaches top_p; never reached: only the
             // maximum survives
-            const int reach = lds_prefixes_below(walk, n, top_p);
+            const float run = wave_serial_prefix(pr, n);
+            const int reach = __popcll(__ballot(lane < n && run < top_p));
             const int at = reach < S ? reach : 0;
-            const float cutoff = walk[at];
+            const float cutoff = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pr), at));
             if (!(live && pr > 0.0f && pr >= cutoff)) pr = 0.0f;
-            __builtin_amdgcn_wave_barrier();
             in_order[lane] = 0.0f;
             __builtin_amdgcn_wave_barrier();
             if (live) in_order[ri] = pr;
             __builtin_amdgcn_wave_barrier();
             po = in_order[lane];
-            const float total = lds_total_in_order(in_order, n);
+            const float total = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_serial_prefix(po, n)), n - 1));
             if (total > 0.0f) po = po / total;
         }
         int chosen = 0;
         if (u > 0.0f) {
-            __builtin_amdgcn_wave_barrier();
-            walk[lane] = po;
-            __builtin_amdgcn_wave_barrier();
-            const int hit = lds_prefixes_below(walk, n, u);  // first i with u <= cumulative
-            chosen = hit < S ? perm[64 + hit] : V - 1;
+            const float run = wave_serial_prefix(po, n);
+            const int hit = __popcll(__ballot(lane < n && run < u));  // first i with u <= cumulative
+            chosen = hit < S ? perm[64 + hit] : (ids ? last_id : V - 1);
         }
         if (tid == 0) ishare[1] = chosen;
     }
+    PTICK(5);
     __syncthreads();
+    PTICK(6);
     return ishare[1];
 }
 

@@ -23,6 +23,7 @@ FLAG_STEPWISE_PROMPT = 2
 FLAG_SMALL_ATTENTION_CHUNKS = 4
 FLAG_CLASSIC_PERSISTENT = 8
 FLAG_XCD_PERSISTENT = 16
+FLAG_ROW_PICKS = 32
 
 
 class DeviceError(RuntimeError):
@@ -52,7 +53,7 @@ class GhSampling(C.Structure):
 
 class GhTiming(C.Structure):
     _fields_ = [("prompt_ms", C.c_float), ("decode_ms", C.c_float), ("prompt_steps", C.c_int32),
-                ("decode_steps", C.c_int32), ("launches_per_step", C.c_int32)]
+                ("decode_steps", C.c_int32), ("launches_per_step", C.c_int32), ("row_picks", C.c_int32)]
 
 
 class GhTokenizerInfo(C.Structure):

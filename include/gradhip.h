@@ -129,6 +129,13 @@ enum { GH_FLAG_SMALL_ATTENTION_CHUNKS = 4 };
 enum { GH_FLAG_CLASSIC_PERSISTENT = 8 };
 enum { GH_FLAG_XCD_PERSISTENT = 16 };
 
+/* In the all-to-all persistent kernel a greedy pick, and a pick with 0 < top_k <= 64,
+ * that follows a step of the same launch is made by every workgroup at once from a
+ * few candidates per workgroup; every other pick by one workgroup from the whole row
+ * of logits.  This flag leaves every pick to the one workgroup, for comparing the two
+ * and for tests. */
+enum { GH_FLAG_ROW_PICKS = 32 };
+
 /* InferenceSession::InferenceSession (inference.cpp:121-148): allocates the
  * paged KV cache (2 * layers * max_len * d_model floats per sequence) and the
  * per-step scratch, and records the step graph. */
@@ -330,6 +337,10 @@ typedef struct gh_timing {
     int32_t prompt_steps;
     int32_t decode_steps;
     int32_t launches_per_step; /* kernel launches (or graph nodes) in one step */
+    /* Persistent engine, since the session was created: picks that one workgroup made from
+     * the whole row of logits.  The others (greedy, or 0 < top_k <= 64, after a step of the
+     * same launch) were made by every workgroup at once from a few candidates per workgroup. */
+    int32_t row_picks;
 } gh_timing;
 gh_status gh_session_last_timing(const gh_session* s, gh_timing* out);
 

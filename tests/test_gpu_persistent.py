@@ -148,6 +148,77 @@ def test_penalty_window_with_a_vocabulary_smaller_than_the_window_needs():
             check_sampled_stream(got[0], ref, rsl, 5, u, opts, f"vocab 100 sampled {penalty} engine {engine}")
 
 
+def test_picks_made_by_every_workgroup_and_the_takeover_by_one(models):
+    """After a step of the same launch a greedy pick, and a pick with 0 < top_k <= 64, is made
+    by every workgroup from a few candidates per workgroup (its largest logit; its four
+    largest and the value of the fifth).  The candidates hold the whole cut only while no
+    workgroup keeps back a value that reaches the k-th largest: otherwise workgroup 0 picks
+    from the row as it does for every other sampler setting.  Both ways must give the
+    checker's stream; `row_picks` says which way a pick went."""
+    cfg = synth.Config(synth.ARCH_GPT2, 4200, 512, 1, 8, 80)  # every workgroup has rows of the logits
+    W, om = make_pair(cfg, 40, std=0.05, norm_noise=0.1)
+    gm = G.Model.from_tensors(cfg, W)
+    prompt = synth.uniform_tokens(9, cfg.vocab, 12)
+    n = 60
+    u = synth.uniforms(n, 13)
+
+    def row_picks(sess):
+        return sess.last_timing()["row_picks"]
+
+    s = G.Session(gm, engine=G.ENGINE_PERSISTENT)
+    # the prompt goes through the batched kernels, so the first pick of a call finds its row
+    # in memory and is workgroup 0's
+    s.generate(prompt, n, G.sampling(greedy=True, repetition_penalty=1.2))
+    assert row_picks(s) == 1
+    opts = (0.8, 40, 0.9, 1.1)
+    ref, rsl = O.generate_sample(om, prompt, u, opts[0], n, opts[3], opts[1], opts[2], want_logits=True)
+    got = s.generate(prompt, n, G.sampling(*opts), uniforms=u)
+    check_sampled_stream(got[0], ref, rsl, 9, u, opts, f"picks by every workgroup {opts}")
+    assert row_picks(s) <= 2 + 3  # a workgroup with five of the forty largest of 4200 is rare
+    before = row_picks(s)
+    s.generate(prompt, n, G.sampling(0.8, 0, 0.9, 1.1), uniforms=u)  # no top-k: the row
+    assert row_picks(s) == before + n
+    before = row_picks(s)
+    small = G.Session(models["llama-d768"][3], engine=G.ENGINE_PERSISTENT)  # 1200 entries: not every workgroup has rows
+    small.generate(prompt % 1200, n, G.sampling(*opts), uniforms=u)
+    assert row_picks(small) == n
+    before = row_picks(s)
+    s.reset()
+    s.prefill(prompt)
+    s.decode(10, G.sampling(greedy=True, repetition_penalty=1.0))  # the first pick reads the prompt pass's row
+    assert row_picks(s) == before + 1
+
+    # A model whose logits do not depend on the context (final norm gain 0: the logit of
+    # token i is beta . E[i]) and whose 24 largest sit in the rows of workgroup 0 (rows
+    # 0..7 of every 2048): no top-k pick can be made from four candidates per workgroup.
+    cfg2 = cfg
+    W2 = synth.make_weights(cfg2, 41, std=0.05)
+    names = [t[0] for t in synth.tensor_specs(cfg2)]
+    beta = synth.normal(cfg2.d_model, 41, 900, 1.0)
+    target = synth.normal(cfg2.vocab, 41, 901, 1.0)
+    crowd = np.concatenate([np.arange(8) + 2048 * w for w in range(3)])
+    target[crowd] = 20.0 + 0.05 * np.arange(len(crowd), dtype=np.float32)
+    W2[names.index("token embedding")] = np.outer(target, beta / float(beta @ beta)).astype(np.float32)
+    W2[names.index("final norm gamma")][:] = 0.0
+    W2[names.index("final norm beta")] = beta.reshape(1, -1).astype(np.float32)
+    om2 = O.Model.from_tensors(cfg2, W2)
+    gm2 = G.Model.from_tensors(cfg2, W2)
+    prompt = synth.uniform_tokens(5, cfg2.vocab, 14)
+    n = 50
+    u = synth.uniforms(n, 15)
+    s = G.Session(gm2, engine=G.ENGINE_PERSISTENT)
+    for opts in ((0.8, 10, 0.9, 1.1), (1.2, 20, 1.0, 1.3)):
+        before = row_picks(s)
+        ref, rsl = O.generate_sample(om2, prompt, u, opts[0], n, opts[3], opts[1], opts[2], want_logits=True)
+        got = s.generate(prompt, n, G.sampling(*opts), uniforms=u)
+        check_sampled_stream(got[0], ref, rsl, 5, u, opts, f"crowded workgroup {opts}")
+        assert set(got[0][5:].tolist()) <= set(crowd.tolist())
+        assert row_picks(s) == before + n  # every pick was handed to workgroup 0
+    ref, rsl = O.generate_greedy(om2, prompt, n, 1.2, want_logits=True)
+    got = s.generate(prompt, n, G.sampling(greedy=True, repetition_penalty=1.2))
+    check_greedy_stream(got[0], ref, rsl, 5, "crowded workgroup greedy")
+
+
 def test_unsupported_shapes_fall_back_or_refuse(models):
     cfg = synth.Config(synth.ARCH_MODERN, 301, 128, 2, 2, 40)
     gm = G.Model.from_tensors(cfg, synth.make_weights(cfg, 1))
