@@ -343,6 +343,13 @@ struct Session {
     hipStream_t stream = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    // Batched greedy decoding without a penalty: the logits launch leaves the largest
+    // value of every run of 16 columns, and a second form of the step opens with the
+    // launch that picks from those and embeds (no pick launch, no embedding launch).
+    float2* best = nullptr;  // [B][best_stride]
+    int best_stride = 0;
+    hipGraph_t graph_fused = nullptr;
+    hipGraphExec_t exec_fused = nullptr;
     hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
 
     float* kv_pool = nullptr;
@@ -431,6 +438,9 @@ struct Session {
         }
         if (exec) (void)hipGraphExecDestroy(exec);
         if (graph) (void)hipGraphDestroy(graph);
+        if (exec_fused) (void)hipGraphExecDestroy(exec_fused);
+        if (graph_fused) (void)hipGraphDestroy(graph_fused);
+        if (best) (void)hipFree(best);
         for (hipEvent_t e : ev)
             if (e) (void)hipEventDestroy(e);
         for (void* p : {static_cast<void*>(kv_pool), static_cast<void*>(page_table),
@@ -591,13 +601,17 @@ static int enqueue_logits(Session& s, bool advance) {
     g.out = s.logits;
     g.out_stride = sh.vocab;
     g.advance = advance ? s.st : nullptr;
+    g.best = s.best;
+    g.best_stride = s.best_stride;
     return modern ? project<PRO_RMSNORM, EPI_STORE>(s, g, s.stream)
                   : project<PRO_LAYERNORM, EPI_STORE>(s, g, s.stream);
 }
 
 // One InferenceSession::step for every sequence (inference.cpp:150-258),
 // enqueued on the session stream.  Returns the number of launches.
-static int enqueue_step(Session& s) {
+// pick_first: the step opens with the greedy pick from what the last logits launch
+// left in s.best (text_gen.cpp:52-60), which also writes the input rows.
+static int enqueue_step(Session& s, bool pick_first = false) {
     const Model& m = *s.m;
     const Shape& sh = m.shape;
     const int d = sh.d_model, F = sh.d_ff(), B = s.B;
@@ -605,8 +619,13 @@ static int enqueue_step(Session& s) {
     hipStream_t st = s.stream;
     int launches = 0;
 
-    hipLaunchKernelGGL(embed_kernel, dim3((d + 255) / 256, B), dim3(256), 0, st, m.E, m.P, s.tok,
-                       s.st, s.x, d);
+    if (pick_first) {
+        hipLaunchKernelGGL(argmax_embed_kernel, dim3(B), dim3(kArgmaxThreads), 0, st, s.best, s.best_stride, s.st,
+                           s.hist, s.hist_stride, s.tok, m.E, m.P, s.x, d);
+    } else {
+        hipLaunchKernelGGL(embed_kernel, dim3((d + 255) / 256, B), dim3(256), 0, st, m.E, m.P, s.tok,
+                           s.st, s.x, d);
+    }
     HIP_CHECK(hipGetLastError());
     launches++;
 
@@ -1030,11 +1049,11 @@ static void check_persist_abort(Session& s) {
     }
 }
 
-static void run_step(Session& s) {
+static void run_step(Session& s, bool pick_first = false) {
     if (s.engine == GH_ENGINE_GRAPH) {
-        HIP_CHECK(hipGraphLaunch(s.exec, s.stream));
+        HIP_CHECK(hipGraphLaunch(pick_first ? s.exec_fused : s.exec, s.stream));
     } else {
-        enqueue_step(s);
+        enqueue_step(s, pick_first);
     }
     s.pos++;
 }
@@ -1056,6 +1075,7 @@ __global__ void set_state_kernel(DevState* st, int pos, int n_hist, int picks) {
     st->pos = pos;
     st->n_hist = n_hist;
     st->picks = picks;
+    st->hist_lead = n_hist - pos;
 }
 
 // tok[b] = hist[b][t]
@@ -1269,6 +1289,13 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
     reset_session(s);
     HIP_CHECK(hipStreamSynchronize(s.stream));
 
+    // The matrix-core logits launch can leave what a greedy pick needs (a batch of at
+    // least two sequences takes it; the wide form and the tiled form both can).
+    if (s.engine != GH_ENGINE_PERSISTENT && s.B >= kMinGemmBatch && gemm_shape_ok(sh.d_model, sh.d_model)) {
+        s.best_stride = (sh.vocab + 15) / 16;
+        dev_alloc(s.best, static_cast<size_t>(s.B) * s.best_stride);
+    }
+
     if (s.engine == GH_ENGINE_PERSISTENT) {
         // nothing to record: one launch runs any number of steps
     } else if (s.engine == GH_ENGINE_GRAPH) {
@@ -1283,6 +1310,19 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
         }
         HIP_CHECK(hipStreamEndCapture(s.stream, &s.graph));
         HIP_CHECK(hipGraphInstantiate(&s.exec, s.graph, nullptr, nullptr, 0));
+        if (s.best) {
+            HIP_CHECK(hipStreamBeginCapture(s.stream, hipStreamCaptureModeThreadLocal));
+            try {
+                enqueue_step(s, true);
+            } catch (...) {
+                hipGraph_t g = nullptr;
+                (void)hipStreamEndCapture(s.stream, &g);
+                if (g) (void)hipGraphDestroy(g);
+                throw;
+            }
+            HIP_CHECK(hipStreamEndCapture(s.stream, &s.graph_fused));
+            HIP_CHECK(hipGraphInstantiate(&s.exec_fused, s.graph_fused, nullptr, nullptr, 0));
+        }
     } else {
         // Count the launches of one step without running it twice: a dry capture.
         HIP_CHECK(hipStreamBeginCapture(s.stream, hipStreamCaptureModeThreadLocal));
@@ -1603,13 +1643,26 @@ static std::pair<int, int> run_decode(Session& s, int max_tokens, const gh_sampl
         if (steps_logged) *steps_logged += steps;
         return {picks, steps};
     }
+    // Greedy without a penalty on the matrix-core path: after the first step of the call
+    // the pick rides at the head of the next step (the logits launch left what it needs).
+    const bool pick_rides = s.best && o.greedy && o.repetition_penalty == 1.0f;
+    if (pick_rides) {
+        hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, s.stream, s.st, s.pos, s.n_hist, s.picks);
+        HIP_CHECK(hipGetLastError());
+    }
     int picks = 0, steps = 0;
     for (int i = 0; i < max_tokens; i++) {
         if (s.n_hist >= s.hist_stride) break;
-        launch_pick(s, o, du, u_stride, seed, true);
+        const bool riding = pick_rides && steps > 0 && s.pos < C;
+        if (riding) {
+            s.n_hist++;
+            s.picks++;
+        } else {
+            launch_pick(s, o, du, u_stride, seed, true);
+        }
         picks++;
         if (s.pos >= C) break;
-        run_step(s);
+        run_step(s, riding);
         steps++;
         if (log) {
             HIP_CHECK(hipMemcpyAsync(log + *steps_logged * BV, s.logits, BV * sizeof(float),

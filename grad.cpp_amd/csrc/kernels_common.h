@@ -17,7 +17,7 @@ struct DevState {
     int pos;     // positions already in the cache (shared by all sequences)
     int n_hist;  // tokens in each sequence's history (prompt + picks)
     int picks;   // picks made so far (index of the next uniform draw)
-    int pad;
+    int hist_lead;  // n_hist - pos when the next pick is made (0 in a decode loop: the pick lands at hist[pos])
 };
 
 // Paged KV cache.  pool is [layers][n_pages][2 (K,V)][heads][page_tokens][head_size];

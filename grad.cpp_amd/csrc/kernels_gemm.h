@@ -282,6 +282,18 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
         const bool has1 = n + 1 < p.N;
         if (e == static_cast<int>(threadIdx.x)) epi_apply<EPI>(p, m, n, v0, v1, has1, first_epi);
         else gemv_epilogue<EPI>(p, m, n, v0, v1, has1);
+        if constexpr (EPI == EPI_STORE) {
+            if (p.best) {
+                // eight neighbouring lanes hold the 16 columns of one row of one tile, in
+                // column order: fold them (an inactive lane's value is never taken)
+                float bv = (has1 && v1 > v0) ? v1 : v0;
+                int bn = (has1 && v1 > v0) ? n + 1 : n;
+                first_max_step<0xB1, 0xF>(bv, bn);
+                first_max_step<0x4E, 0xF>(bv, bn);
+                first_max_step<0x141, 0xF>(bv, bn);
+                if ((e & 7) == 0) p.best[static_cast<size_t>(m) * p.best_stride + (n >> 4)] = make_float2(bv, __int_as_float(bn));
+            }
+        }
     }
 }
 
@@ -452,6 +464,17 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const GemvParams p, int 
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(v0), rs_o, e_live && n < p.N ? o : kPastEnd, 0, 0);
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(v1), rs_o,
                                                       e_live && n + 1 < p.N ? o + 4u : kPastEnd, 0, 0);
+                if (p.best) {
+                    // eight neighbouring lanes hold the tile's 16 columns of one row, in column order
+                    const bool has1 = n + 1 < p.N;
+                    float bv = n < p.N ? ((has1 && v1 > v0) ? v1 : v0) : -INFINITY;
+                    int bn = (has1 && v1 > v0) ? n + 1 : n;
+                    first_max_step<0xB1, 0xF>(bv, bn);
+                    first_max_step<0x4E, 0xF>(bv, bn);
+                    first_max_step<0x141, 0xF>(bv, bn);
+                    if ((e & 7) == 0 && e_live && n < p.N)
+                        p.best[static_cast<size_t>(em) * p.best_stride + tile] = make_float2(bv, __int_as_float(bn));
+                }
             }
             __syncthreads();  // red is rewritten by the next tile
         }

@@ -41,6 +41,12 @@ struct GemvParams {
     // rows_per_seq == 0: one row per sequence, all at st->pos (a decode step).
     int rows_per_seq;
     int pos_base;
+    // EPI_STORE on the matrix-core kernels only: when set, the largest output of every
+    // row in every run of 16 columns and its first column, best[row * best_stride +
+    // column / 16] = {value, column as int bits}: what an arg-max over the row needs
+    // (text_gen.cpp:52-60) without reading the row back.
+    float2* best;
+    int best_stride;
 };
 
 // What the epilogue of one pair of outputs (row, row + 1) of input row b needs

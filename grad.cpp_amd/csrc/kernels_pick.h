@@ -988,4 +988,60 @@ __global__ __launch_bounds__(kPickThreads) void pick_kernel(const PickParams p) 
     }
 }
 
+// The greedy pick without a penalty for every sequence of a batched step, and the
+// embedding of what it picked, in one launch (text_gen.cpp:52-60, inference.cpp:159-182).
+// The logits launch left the largest value and first column of every run of 16 columns
+// of every row; one workgroup per sequence takes the first maximum of those, records
+// the token in the history and writes the step's input row.
+constexpr int kArgmaxThreads = 256;
+
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_embed_kernel(const float2* __restrict__ best, int n16,
+                                                                      const DevState* st, int* hist, int hist_stride,
+                                                                      int* tok, const float* __restrict__ E,
+                                                                      const float* __restrict__ P, float* x, int d) {
+    __shared__ float wv[kArgmaxThreads / 64];
+    __shared__ int wi[kArgmaxThreads / 64];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int pos = st->pos, at = st->pos + st->hist_lead;
+    const float2* row = best + static_cast<size_t>(b) * n16;
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int i0 = 0; i0 < n16; i0 += 4 * kArgmaxThreads) {
+        float2 e[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) e[q] = row[min(i0 + q * kArgmaxThreads + tid, n16 - 1)];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            // a thread's runs come in rising column order: the first maximum stays
+            if (i0 + q * kArgmaxThreads + tid < n16 && e[q].x > bv) {
+                bv = e[q].x;
+                bi = __float_as_int(e[q].y);
+            }
+        }
+    }
+    wave_first_max(bv, bi);
+    if ((tid & 63) == 0) {
+        wv[tid >> 6] = bv;
+        wi[tid >> 6] = bi;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kArgmaxThreads / 64; w++) {
+        if (w == 0 || wv[w] > bv || (wv[w] == bv && wi[w] < bi)) {
+            bv = wv[w];
+            bi = wi[w];
+        }
+    }
+    const int chosen = bi == 0x7FFFFFFF ? 0 : bi;
+    if (tid == 0) {
+        hist[static_cast<size_t>(b) * hist_stride + at] = chosen;  // tokens.push_back(next)
+        tok[b] = chosen;
+    }
+    for (int j = tid; j < d; j += kArgmaxThreads) {
+        float v = E[static_cast<size_t>(chosen) * d + j];
+        if (P) v += P[static_cast<size_t>(pos) * d + j];
+        x[static_cast<size_t>(b) * d + j] = v;
+    }
+}
+
 }  // namespace gh

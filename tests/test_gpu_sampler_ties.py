@@ -20,6 +20,9 @@ CASES = {
     "small": (synth.Config(synth.ARCH_MODERN, 600, 128, 2, 2, 40), 37),       # groups of ~16 tokens
     "wide-groups": (synth.Config(synth.ARCH_GPT2, 1500, 128, 2, 2, 40), 3),   # groups of 500 tokens
     "persistent": (synth.Config(synth.ARCH_MODERN, 1200, 768, 2, 12, 48), 50),  # groups of 24, one-launch engine
+    # every workgroup of the one-launch engine has rows of the logits: top-k picks are made from four
+    # candidates per workgroup, and ties at the cut hand the pick back to the whole row
+    "persistent-wide": (synth.Config(synth.ARCH_MODERN, 4096, 768, 1, 12, 40), 500),
 }
 SAMPLERS = [
     (1.0, 40, 0.9, 1.0),   # the threshold group straddles k = 40
@@ -79,3 +82,29 @@ def test_greedy_picks_the_lowest_tied_index(models, name):
     got, _ = G.Session(gm).generate(prompt, n, G.sampling(greedy=True, repetition_penalty=1.0), want_logits=True)
     check_greedy_stream(got[0], ref, rsl, len(prompt), name)
     assert np.all(np.asarray(ref[len(prompt):]) < distinct)  # always the first copy of the winning row
+
+
+@pytest.mark.parametrize("engine", [G.ENGINE_GRAPH, G.ENGINE_EAGER])
+@pytest.mark.parametrize("batch", [16, 32, 64])
+def test_batched_greedy_picks_the_lowest_tied_index(batch, engine):
+    """Batched greedy decoding without a penalty takes its pick from what the logits launch
+    leaves per run of 16 columns (the few-rows kernel at 16 and 32 sequences, the tiled one
+    at 64) and embeds it in the same launch: ties across runs, tiles and workgroups must
+    still go to the lowest index, for every sequence."""
+    cfg = synth.Config(synth.ARCH_GPT2, 9000, 512, 1, 8, 24)
+    distinct = 7
+    W, om, gm = tied_model(cfg, distinct, 78)
+    prompts = np.stack([synth.uniform_tokens(4, cfg.vocab, 33, stream=b) for b in range(batch)])
+    n = cfg.max_len - 4 + 3  # runs into the capacity rule: the last pick has no step behind it
+    s = G.Session(gm, batch=batch, engine=engine)
+    got = s.generate(prompts, n, G.sampling(greedy=True, repetition_penalty=1.0))
+    for b in range(0, batch, max(1, batch // 8)):
+        ref, rsl = O.generate_greedy(om, prompts[b], n, 1.0, want_logits=True)
+        check_greedy_stream(got[b], ref, rsl, 4, f"batch {batch} sequence {b}")
+        assert np.all(np.asarray(ref[4:]) < distinct)
+    # the same through decode calls that continue one context
+    s.reset()
+    s.prefill(prompts)
+    a = s.decode(5, G.sampling(greedy=True, repetition_penalty=1.0))
+    b2 = s.decode(n - 5, G.sampling(greedy=True, repetition_penalty=1.0))
+    np.testing.assert_array_equal(np.concatenate([prompts, a, b2], axis=1), got)
