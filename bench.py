@@ -35,8 +35,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # number of steps, so the ratio carries over to other launch lengths; the summary named
 # here holds the commands and the raw counts.
 PMC_SOURCE = "profiles/persist_decode_kernel_c2_batch1.md"
-PMC_FETCH_BYTES_PER_LAUNCH = 31_352_668 * 2048  # counter reads 1 per 2 KiB fetched
-PMC_WRITE_BYTES_PER_LAUNCH = 540_302 * 1024     # counter reads 1 per KiB written
+PMC_FETCH_BYTES_PER_LAUNCH = 31_362_617 * 2048  # counter reads 1 per 2 KiB fetched
+PMC_WRITE_BYTES_PER_LAUNCH = 556_358 * 1024     # counter reads 1 per KiB written
 PMC_ALGORITHMIC_BYTES_PER_LAUNCH = 63_406_751_744  # step_bytes() summed over that launch
 
 
