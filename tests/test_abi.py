@@ -43,7 +43,7 @@ def test_struct_layouts_match_the_header():
     assert C.sizeof(G.GhConfig) == 48 and G.GhConfig.tokenizer_hash.offset == 40
     assert C.sizeof(G.GhSessionOpts) == 20
     assert C.sizeof(G.GhSampling) == 20
-    assert C.sizeof(G.GhTiming) == 20
+    assert C.sizeof(G.GhTiming) == 24 and G.GhTiming.row_picks.offset == 20
 
 
 def test_host_logic_runs_without_a_gpu():
