@@ -60,15 +60,44 @@ def test_noalloc_pick_equals_session_pick_twice_in_a_row():
     G.device_info()  # the documented set-up call: looks the scratch array up on this device
     big = _case(torch, synth.Config(synth.ARCH_MODERN, 50257, 128, 2, 2, 32), 900, 3, 12)
     small = _case(torch, synth.Config(synth.ARCH_GPT2, 777, 128, 2, 2, 32), 910, 1, 9)
+    torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]  # hipMemGetInfo: the device's own count, whoever allocates
     got_big = _run(torch, *[big[0]], *big[2:])
     got_small = _run(torch, *[small[0]], *small[2:])  # smaller rows over the first call's leftovers
     got_big2 = _run(torch, *[big[0]], *big[2:])
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     for i in range(len(OPTIONS)):
         assert np.array_equal(got_big[i], big[1][i]), (OPTIONS[i], got_big[i], big[1][i])
         assert np.array_equal(got_small[i], small[1][i]), (OPTIONS[i], got_small[i], small[1][i])
         assert np.array_equal(got_big2[i], big[1][i])
+
+
+def test_noalloc_pick_under_stream_capture():
+    """The callers the entry point is for: a stream under capture in global mode, where an
+    allocation, a free or a wait inside a call ends the capture with an error.  The
+    captured picks are replayed three times with eager work between the replays and must
+    be the session's every time."""
+    torch = _torch_on_the_loaded_runtime()
+    G.device_info()
+    dev, want, batch, vocab, plen = _case(torch, synth.Config(synth.ARCH_MODERN, 5000, 128, 2, 2, 32), 930, 2, 11)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        for i, o in enumerate(OPTIONS):
+            G.pick_noalloc(dev["logits"].data_ptr(), batch, vocab, dev["hist"].data_ptr(), plen, plen,
+                           G.sampling(**o), dev["out"][i].data_ptr(), uniforms_ptr=dev["u"].data_ptr(),
+                           stream=side.cuda_stream)
+    for _ in range(3):
+        dev["out"].fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = dev["out"].cpu().numpy()
+        for i in range(len(OPTIONS)):
+            assert np.array_equal(got[i], want[i]), (OPTIONS[i], got[i], want[i])
 
 
 def test_noalloc_pick_philox_draws_and_limits():
