@@ -386,7 +386,6 @@ struct Session {
     size_t persist_lds = 0;
     // ... its XCD-sharded form (kernels_xcd.h)
     bool xcd = false;         // the kernel and its buffers are ready
-    bool xcd_always = false;  // GH_FLAG_XCD_PERSISTENT: every launch takes it
     bool xcd_row_lds = false;
     bool row_picks_only = false;  // GH_FLAG_ROW_PICKS
     Cell* xcells = nullptr;
@@ -742,11 +741,13 @@ static PersistKernel persist_kernel_for(const Shape& sh, bool row_lds, bool feed
 
 // ---- the XCD-sharded form of the persistent kernel (kernels_xcd.h)
 
-// First position of a launch from which the XCD-sharded kernel is the default.  Per
-// token on one box, Llama block d768 L8 V16000, greedy: positions 33..256 152 us against
-// 113 for the all-to-all kernel, 257..1024 184 / 154, 1024..1280 203 / 206, 1536..1792
-// 219 / 243, 2048..2304 235 / 281, 3072..3328 267 / 356.
-constexpr int kXcdFromPosition = 1024;
+// The XCD-sharded kernel runs only where GH_FLAG_XCD_PERSISTENT asks for it.  It used to
+// be the default for launches that start at position 1024 or later, where it spreads a
+// head's context over the workgroups of an XCD; since the all-to-all kernel shares a
+// head's long context among idle workgroups itself it is the faster one at every
+// position.  Per token on one box, Llama block d768 L8 V16000, greedy, XCD-sharded /
+// all-to-all: positions 256..512 168 / 132, 512..768 178 / 144, 1024..1280 196 / 149,
+// 2048..2304 228 / 156, 3072..3328 259 / 160, 3800..4056 277 / 162.
 
 using XcdKernel = void (*)(const XcdParams);
 
@@ -1002,9 +1003,7 @@ static void persist_run(Session& s, int n_prompt, int n_steps, int n_picks, bool
     k.work_stride = s.work_stride;
     k.sort_cap = kPickWorkFloats;
 
-    // The XCD-sharded kernel wins where attention is long (it spreads a head's context over
-    // the workgroups of an XCD): launches that start deep in the context take it.
-    if (s.xcd && (s.xcd_always || s.pos >= kXcdFromPosition)) {
+    if (s.xcd) {
         XcdParams x{};
         x.b = p;
         x.gm = m.xcd_geom;
@@ -1206,6 +1205,9 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
             // leave for a pick each of them makes itself: nine planes of one cell per
             // workgroup and a stop word
             s.cells_count = 6 * d + F + 2 + 9 * static_cast<size_t>(s.persist_grid) + 1;
+            // and, from an even index, what the workgroups that share a head's long context
+            // leave for the head's own: up to fifteen shares of 66 cells for each of up to 16 heads
+            s.cells_count = ((s.cells_count + 1) & ~static_cast<size_t>(1)) + 16 * 15 * 66;
             dev_alloc(s.cells, s.cells_count);
             // Rows of the cache written earlier in a launch by other workgroups are read
             // with ordinary loads.  That is sound only because a row is never read before
@@ -1243,8 +1245,7 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
             // compute units, and a ring of a power-of-two size beside the work area
             // (workgroup 0's ring is smaller when the pick keeps its row in LDS).
             XcdGeom gm;
-            const bool xcd_wanted = (o.flags & GH_FLAG_XCD_PERSISTENT) != 0
-                                    || ((o.flags & GH_FLAG_CLASSIC_PERSISTENT) == 0 && sh.max_len > kXcdFromPosition);
+            const bool xcd_wanted = (o.flags & GH_FLAG_XCD_PERSISTENT) != 0;
             if ((o.flags & GH_FLAG_XCD_PERSISTENT) != 0 && (o.flags & GH_FLAG_CLASSIC_PERSISTENT) != 0)
                 throw ApiError{GH_ERR_INVALID_ARGUMENT, "GH_FLAG_CLASSIC_PERSISTENT and GH_FLAG_XCD_PERSISTENT exclude each other"};
             if (xcd_wanted && prop.multiProcessorCount == kXcds * kWgPerXcd && xcd_geometry(sh, gm)
@@ -1269,7 +1270,6 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
                 if (ring >= 64 * 1024) {
                     xcd_build_stream(m);
                     s.xcd = true;
-                    s.xcd_always = (o.flags & GH_FLAG_XCD_PERSISTENT) != 0;
                     s.xcd_all_slices = (o.flags & GH_FLAG_SMALL_ATTENTION_CHUNKS) != 0;
                     s.xcd_ring_units = static_cast<unsigned>(ring / kXcdUnit);
                     s.xcd_ring_units_wg0 = static_cast<unsigned>(ring0 / kXcdUnit);

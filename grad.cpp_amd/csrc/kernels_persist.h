@@ -89,7 +89,9 @@ struct PersistParams {
     // FFN hidden [F], the picked token [1] (+ 1 unused), then what the workgroups leave for
     // a pick that each of them makes itself: planes of one cell per workgroup (greedy:
     // largest logit, its index; top-k: four values, four indices, the fifth value) and
-    // the host's stop request as workgroup 0 read it [1].  The kernel addresses them from the one
+    // the host's stop request as workgroup 0 read it [1]; then, from an even index, the
+    // shares of a head's attention that other workgroups computed [16 heads][15][66].  The
+    // kernel addresses them from the one
     // base: eight pointers held through the whole token loop are sixteen scalar
     // registers that would otherwise be parked in vector lanes and fetched back.
     Cell* cells;
@@ -394,6 +396,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
     constexpr int D = KD * 256, F = KF * 256, HS = 64;
     constexpr int PRO = MODERN ? PRO_RMSNORM : PRO_LAYERNORM;
     constexpr int RL = 8;  // logits rows per wavefront item
+    // Beyond kAttnShareFrom positions a head's attention is shared by several workgroups,
+    // kAttnShare positions each: what a workgroup's eight wavefronts take in one batch of 32.
+    // (One workgroup up to 512 positions: 256..512 ran at 132 us per token alone and 138 in two shares.)
+    constexpr int kAttnShareFrom = 512, kAttnShare = 256, kAttnMaxShares = 16;
     float* xs = lds;                      // [D] residual stream of this step
     float* vin = lds + D;                 // [max(D, F)] attention output / FFN hidden
     float* ascr = vin + (F > D ? F : D);  // attention scratch: q, k, v of the head + wave partials
@@ -633,17 +639,31 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             }
             stamp();
 
-            // ===== phase B: attention of one head per workgroup (inference.cpp:211-225)
-            if (wg < H) {
-                const int hd = wg;
+            // ===== phase B: attention of one head per workgroup (inference.cpp:211-225).
+            // One compute unit fetches a head's cached rows at about 100 GB/s, which is what
+            // a long context costs: beyond kAttnShareFrom positions the context of a head is
+            // cut into shares of at most kAttnShare positions, the last (with the new position)
+            // for the head's own workgroup and the others for the workgroups 16, 32, ... places
+            // further on, which are idle in this phase.  They need q only, leave (maximum, sum,
+            // 64 weighted sums) in cells, and the head's workgroup folds the shares in a fixed order.
+            const int ctx = pos + 1;
+            const int n_shares =
+                ctx <= kAttnShareFrom ? 1 : min(kAttnMaxShares, (ctx + kAttnShare - 1) / kAttnShare);  // uniform
+            const bool head_wg = wg < H;
+            const bool share_wg = !head_wg && (wg & 15) < H && (wg >> 4) < n_shares;
+            if (head_wg || share_wg) {
+                const int hd = wg & 15;
+                const int share = head_wg ? n_shares - 1 : (wg >> 4) - 1;
                 float* qkv = ascr;         // [3][64]: q, key and value of the current position
                 float* part = ascr + 192;  // [waves][4 lane groups][68]: m, l, pad, pad, acc[64]
-                const int ctx = pos + 1;
-                // positions are dealt to the wavefronts in runs of `chunk` (a multiple of 4),
-                // walked 32 at a time
-                const int chunk = (((ctx + kPersistWaves - 1) / kPersistWaves) + 3) & ~3;
+                // this workgroup's positions [lo, hi); they are dealt to the wavefronts in
+                // runs of `chunk` (a multiple of 4), walked 32 at a time
+                const int span = (((ctx + n_shares - 1) / n_shares) + 3) & ~3;
+                const int lo = share * span, hi = min(ctx, lo + span);
+                const int chunk = (((hi - lo + kPersistWaves - 1) / kPersistWaves) + 3) & ~3;
                 const int sub = lane >> 4, dl = lane & 15;
-                const int t0 = wave * chunk;
+                const int t0 = lo + wave * chunk;
+                Cell* share_cells = p.cells + ((6 * D + F + 2 + 9 * G + 2) & ~1);  // [H][15][66]
                 // Cached rows do not depend on this step's q: the first 32 positions of
                 // the run are fetched before waiting for q (all of it for contexts <= 256).
                 const float* pool = p.kv.pool;
@@ -653,19 +673,20 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                     const int tt = t0 + it * 4 + sub;
                     k4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
                     v4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (it * 4 < chunk && tt < pos) {
+                    if (it * 4 < chunk && tt < min(pos, hi)) {
                         const unsigned ko = static_cast<unsigned>(kv_at(l, 0, hd, tt)) + dl * 4;
                         const unsigned vo = static_cast<unsigned>(kv_at(l, 1, hd, tt)) + dl * 4;
                         k4[it] = *reinterpret_cast<const float4*>(pool + ko);
                         v4[it] = *reinterpret_cast<const float4*>(pool + vo);
                     }
                 }
-                // q, new key, new value of this head: one wait for all three
+                // q, new key, new value of this head: one wait for all three (a workgroup with
+                // a share of older positions needs q alone)
                 {
                     const unsigned t = tag_of(l, 0);
                     unsigned spins = 0;
                     bool failed = false;
-                    if (tid < 96) {
+                    if (tid < (head_wg ? 96 : 32)) {
                         const int seg = tid >> 5, j = (tid & 31) * 2;
                         const Cell* src = (seg == 0 ? (p.cells + 2 * D) : seg == 1 ? (p.cells + 3 * D) : (p.cells + 4 * D)) + hd * HS;
                         const __amdgpu_buffer_rsrc_t rs = make_buffer(src, HS * 8u);
@@ -702,7 +723,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                             const int tt = t0 + batch * 32 + it * 4 + sub;
                             k4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
                             v4[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-                            if (batch * 32 + it * 4 < chunk && tt < pos) {
+                            if (batch * 32 + it * 4 < chunk && tt < min(pos, hi)) {
                                 const unsigned ko = static_cast<unsigned>(kv_at(l, 0, hd, tt)) + dl * 4;
                                 const unsigned vo = static_cast<unsigned>(kv_at(l, 1, hd, tt)) + dl * 4;
                                 k4[it] = *reinterpret_cast<const float4*>(pool + ko);
@@ -721,7 +742,7 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                             v4[it] = reinterpret_cast<const float4*>(qkv + 128)[dl];
                         }
                         const float sdot = row16_sum(dot4(q4, k4[it]));
-                        sc[it] = (in_run && tt < ctx) ? sdot * 0.125f : -INFINITY;  // 1/sqrt(64)
+                        sc[it] = (in_run && tt < hi) ? sdot * 0.125f : -INFINITY;  // 1/sqrt(64)
                     }
                     float mb = sc[0];
 #pragma unroll
@@ -783,11 +804,10 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                     }
                 }
                 __syncthreads();
+                float M = -INFINITY, Lsum = 0.0f, o = 0.0f;
                 if (tid < HS) {
-                    float M = -INFINITY;
 #pragma unroll
                     for (int w8 = 0; w8 < kPersistWaves; w8++) M = fmaxf(M, part[w8 * 68]);
-                    float Lsum = 0.0f, o = 0.0f;
                     // one exponential per lane (wavefront lane % 8's), read across by all
                     static_assert(kPersistWaves == 8, "lane % 8 picks a wavefront");
                     const float fmine = expf(part[(tid & 7) * 68] - M);  // 0 for wavefronts without positions
@@ -797,6 +817,37 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
                         Lsum += part[w8 * 68 + 1] * f;
                         o += part[w8 * 68 + 4 + tid] * f;
                     }
+                }
+                if (share_wg) {
+                    // this share's maximum, sum and weighted sums, for the head's workgroup
+                    if (tid < HS) {
+                        Cell* mine_c = share_cells + (hd * (kAttnMaxShares - 1) + share) * 66;
+                        const unsigned t = tag_of(l, 5);
+                        cell_put(mine_c + 2 + tid, o, t);
+                        if (tid == 0) {
+                            cell_put(mine_c, M, t);
+                            cell_put(mine_c + 1, Lsum, t);
+                        }
+                    }
+                } else if (n_shares > 1) {
+                    // the other shares, then the fold in share order with this one last
+                    __syncthreads();  // part[] is read; it takes the shares now
+                    if (!gather_cells(share_cells + hd * (kAttnMaxShares - 1) * 66, (n_shares - 1) * 66, tag_of(l, 5), part, p)) return;
+                    if (tid < HS) {
+                        float Mall = M;
+                        for (int j = 0; j < n_shares - 1; j++) Mall = fmaxf(Mall, part[j * 66]);
+                        float Lall = 0.0f, oall = 0.0f;
+                        for (int j = 0; j < n_shares - 1; j++) {
+                            const float f = expf(part[j * 66] - Mall);
+                            Lall += part[j * 66 + 1] * f;
+                            oall += part[j * 66 + 2 + tid] * f;
+                        }
+                        const float f = expf(M - Mall);
+                        Lall += Lsum * f;
+                        oall += o * f;
+                        cell_put((p.cells + 5 * D) + hd * HS + tid, oall * (1.0f / Lall), tag_of(l, 1));
+                    }
+                } else if (tid < HS) {
                     cell_put((p.cells + 5 * D) + hd * HS + tid, o * (1.0f / Lsum), tag_of(l, 1));
                 }
                 __syncthreads();

@@ -121,11 +121,12 @@ enum { GH_FLAG_STEPWISE_PROMPT = 2 };
 enum { GH_FLAG_SMALL_ATTENTION_CHUNKS = 4 };
 
 /* The persistent engine has two kernels for the Llama block at d_model 768: one in
- * which every phase of a layer is exchanged among all 256 workgroups, and one that
- * splits a layer over the eight XCDs and streams the weights through LDS.  By
- * default a launch that starts at or beyond position 1024 takes the second (its
- * attention is spread over all workgroups of an XCD) and every other launch the
- * first.  These two flags pin the choice, for comparing the kernels and for tests. */
+ * which every phase of a layer is exchanged among all 256 workgroups (and a head's
+ * context beyond 512 positions is shared among idle workgroups), and one that splits a
+ * layer over the eight XCDs and streams the weights through LDS.  The first is the
+ * faster at every context and the default; GH_FLAG_XCD_PERSISTENT selects the second
+ * for every launch of the session (for comparing the kernels and for tests), and
+ * GH_FLAG_CLASSIC_PERSISTENT names the default explicitly.  The two exclude each other. */
 enum { GH_FLAG_CLASSIC_PERSISTENT = 8 };
 enum { GH_FLAG_XCD_PERSISTENT = 16 };
 

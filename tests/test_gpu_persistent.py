@@ -125,6 +125,43 @@ def test_long_context_runs_of_more_than_64_positions_per_wavefront():
             s.step([int(t)])
 
 
+@pytest.mark.parametrize("arch,d,heads,max_len,start", [
+    (synth.ARCH_MODERN, 768, 12, 1800, 1480),  # 6, 7, 8 shares
+    (synth.ARCH_GPT2, 1024, 16, 640, 470),     # every workgroup of the first 16 has a head; 1 share, then 3
+    (synth.ARCH_MODERN, 768, 12, 4096, 3800),  # 15, then 16 shares: the largest context
+])
+def test_long_context_shared_by_several_workgroups(arch, d, heads, max_len, start):
+    """Beyond 512 positions the context of a head is cut into shares of at most 256 positions: the
+    head's workgroup keeps the last one and folds in what the workgroups 16, 32, ... places
+    further on leave for it.  The all-to-all kernel is pinned, so that it runs past the
+    position where the other kernel would take over."""
+    cfg = synth.Config(arch, 400, d, 1, heads, max_len)
+    W, om = make_pair(cfg, 29, std=0.05, norm_noise=0.1)
+    gm = G.Model.from_tensors(cfg, W)
+    s = G.Session(gm, engine=G.ENGINE_PERSISTENT, flags=G.FLAG_CLASSIC_PERSISTENT)
+    shuffled = G.Session(gm, engine=G.ENGINE_PERSISTENT, flags=G.FLAG_CLASSIC_PERSISTENT, shuffle_pages=True,
+                         page_tokens=8)
+    osess = O.Session(om)
+    toks = synth.uniform_tokens(cfg.max_len, cfg.vocab, 9)
+    for t in toks[:start]:
+        ref = osess.step(int(t))
+    assert_logits_close(s.prefill(toks[None, :start])[0], ref, 1e-4, f"after a {start}-token prompt")
+    shuffled.prefill(toks[None, :start])
+    for i, t in enumerate(toks[start:]):
+        ref = osess.step(int(t))
+        a = s.step([int(t)])[0]
+        assert np.array_equal(a, shuffled.step([int(t)])[0])  # page placement does not matter
+        if i % 10 == 0 or start + i in (319, 320, 321, 511, 512, 513, 1535, 1536, 1537, 3839, 3840, 3841) or i >= len(toks) - start - 3:
+            assert_logits_close(a, ref, 1e-4, f"shared attention position {start + i}")
+    # one launch across a change of the number of shares, greedy against the checker
+    g = G.Session(gm, engine=G.ENGINE_PERSISTENT, flags=G.FLAG_CLASSIC_PERSISTENT)
+    g.prefill(toks[None, :start])
+    n = min(120, cfg.max_len - start)
+    got = g.decode(n, G.sampling(greedy=True, repetition_penalty=1.0))[0]
+    ref, rsl = O.generate_greedy(om, toks[:start], n, 1.0, want_logits=True)
+    check_greedy_stream(np.concatenate([toks[:start], got]), ref, rsl, start, "shared attention greedy run")
+
+
 def test_penalty_window_with_a_vocabulary_smaller_than_the_window_needs():
     """The penalty window (50 tokens) is counted by one wavefront in registers.  With a
     vocabulary of 100 fewer than 50 threads have a part of the row to load: the count must
