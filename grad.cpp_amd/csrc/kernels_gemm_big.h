@@ -1,9 +1,11 @@
 // Projections over many rows (a prompt pass: hundreds to tens of thousands of
 // token rows): C[M,N] = A[M,K] . Wt[N,K]^T on the fp32 matrix cores with the
 // classic compute-bound tiling — one workgroup owns a 128 x 128 tile of C, its
-// four wavefronts 64 x 64 each (16 accumulator tiles of 16 x 16), and A and W
-// travel through LDS in K-steps of 16, double buffered, fetched with
-// row-contiguous 16-byte loads.  The 64-row decode kernel (gemm16_kernel) is
+// four wavefronts 64 x 64 each (four accumulator tiles of 32 x 32, products
+// v_mfma_f32_32x32x2_f32: 730 k tok/s on the 16 x 1536-token prompt pass against
+// 711 k with sixteen 16 x 16 tiles and the 16x16x4 product, same LDS reads, half
+// the product instructions), and A and W travel through LDS in K-steps of 16,
+// double buffered, fetched with row-contiguous 16-byte loads.  The 64-row decode kernel (gemm16_kernel) is
 // bound by latency and wants many small tiles; here the arithmetic is the bound
 // and every fetched element is reused 64 times from LDS.
 //
@@ -34,7 +36,6 @@ __global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p
     float* row_scale = lds_big + kBigTile * kBigCLd;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;  // 64 x 64 quadrant of the tile
-    const int j = lane & 15, g = lane >> 4;
     const int m_tile = blockIdx.x / n_tiles, n_tile = blockIdx.x - m_tile * n_tiles;
     const int m0 = m_tile * kBigTile, n0 = n_tile * kBigTile;
     const int K = p.K;
@@ -48,11 +49,15 @@ __global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p
     const float* g_src = RMS ? p.gamma + fc * 4 : nullptr;
     const int stash_at = fr * kBigLd + fc * 4;  // this thread's float4 slot in a staged tile (second row: + 64 rows)
 
-    v4f acc[4][4];
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    v16f acc32[2][2];
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < 2; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) acc[a][b] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc32[a][b][r] = 0.0f;
+    const int i32 = lane & 31, h32 = lane >> 5;
     float ss0 = 0.0f, ss1 = 0.0f;
 
     float4 ra0, ra1, rw0, rw1, rg = make_float4(1.f, 1.f, 1.f, 1.f);
@@ -89,35 +94,41 @@ __global__ __launch_bounds__(kBigThreads) void gemm128_kernel(const GemvParams p
         }
         const float* as = stage + buf * (2 * kBigTile * kBigLd) + (wm * 64) * kBigLd;
         const float* ws = stage + buf * (2 * kBigTile * kBigLd) + kBigTile * kBigLd + (wn * 64) * kBigLd;
-        float4 fa[4], fb[4];
+        // 32 x 32 x 2 products: lane (row i32, half h32) brings k = 4 h32 + e (+ 8 q) to product e of
+        // round q, for A and W alike, so every k of the step is multiplied once
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            fa[t] = *reinterpret_cast<const float4*>(as + (t * 16 + j) * kBigLd + g * 4);
-            fb[t] = *reinterpret_cast<const float4*>(ws + (t * 16 + j) * kBigLd + g * 4);
-        }
+        for (int q = 0; q < 2; q++) {
+            float4 fa[2], fb[2];
 #pragma unroll
-        for (int a = 0; a < 4; a++)
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].x, fb[b].x, acc[a][b], 0, 0, 0);
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].y, fb[b].y, acc[a][b], 0, 0, 0);
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].z, fb[b].z, acc[a][b], 0, 0, 0);
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[a].w, fb[b].w, acc[a][b], 0, 0, 0);
+            for (int t = 0; t < 2; t++) {
+                fa[t] = *reinterpret_cast<const float4*>(as + (t * 32 + i32) * kBigLd + q * 8 + h32 * 4);
+                fb[t] = *reinterpret_cast<const float4*>(ws + (t * 32 + i32) * kBigLd + q * 8 + h32 * 4);
             }
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++) {
+                    acc32[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a].x, fb[b].x, acc32[a][b], 0, 0, 0);
+                    acc32[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a].y, fb[b].y, acc32[a][b], 0, 0, 0);
+                    acc32[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a].z, fb[b].z, acc32[a][b], 0, 0, 0);
+                    acc32[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a].w, fb[b].w, acc32[a][b], 0, 0, 0);
+                }
+        }
         if (s + 1 < steps) GH_BIG_STASH(buf ^ 1)
         __syncthreads();
     }
 #undef GH_BIG_FETCH
 #undef GH_BIG_STASH
 
-    // finished tile -> LDS (accumulator layout: lane holds column j, rows 4g + r)
+    // finished tile -> LDS (accumulator layout: lane holds column i32, rows 8 (r / 4) + 4 h32 + r % 4)
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < 2; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++)
+        for (int b = 0; b < 2; b++)
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-                ctile[(wm * 64 + a * 16 + 4 * g + r) * kBigCLd + wn * 64 + b * 16 + j] = acc[a][b][r];
+            for (int r = 0; r < 16; r++)
+                ctile[(wm * 64 + a * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3)) * kBigCLd + wn * 64 + b * 32 + i32] =
+                    acc32[a][b][r];
     if (RMS) {
         // the four threads that fetched a row hold its partial sums of squares
         float v0 = ss0, v1 = ss1;
