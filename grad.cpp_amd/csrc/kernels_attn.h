@@ -564,4 +564,193 @@ __global__ __launch_bounds__(256) void attn_prefill64_kernel(const PrefillAttnPa
     }
 }
 
+// The same attention for longer prompts: one workgroup = 128 consecutive queries of one
+// (sequence, head), 32 per wavefront, on the 32 x 32 x 2 form of the fp32 matrix product.
+// Against the 64-query kernel above a staged K/V tile serves twice as many queries and an
+// operand read from LDS twice as many products, the next tile's rows travel from memory
+// into registers while the current tile is multiplied, and the workgroups with the most
+// keys in front of them are dealt first.  Both products are again formed transposed:
+//   S^T[key][query] = K . Q^T : a lane holds one query (lane % 32) and, of every block of
+//   32 keys, keys 8 (r / 4) + 4 (lane / 32) + r % 4 for r = 0..15,
+// which is the B-operand layout of O^T[dim][query] += V^T . P^T when K-slot lane / 32 of
+// product step e of key group c stands for key 8 c + 4 (lane / 32) + e on both operands.
+// The online softmax is inference.cpp:211-225 taken a tile at a time.
+// What bounds it: on this part nothing else issues on a SIMD while an fp32 matrix product
+// runs (a wavefront's ordinary arithmetic takes as long beside another wavefront's
+// v_mfma_f32_32x32x2_f32 chain as the two take one after the other), so the softmax
+// arithmetic (about 700 vector instructions per wavefront and tile, 430 of them the 33
+// precise exponentials) adds to the 128 products of a tile instead of hiding behind them:
+// 16 x 12 heads x 1536 tokens take 0.86 ms, of which the products alone are 0.39.
+typedef float attn_v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill128_kernel(const PrefillAttnParams p) {
+    constexpr int HS = 64, TILE = 64, QB = 128, LDK = HS + 4, LDV = TILE + 4;
+    __shared__ float Ks[TILE * LDK];  // [key][dim]
+    __shared__ float Vt[HS * LDV];    // [dim][key]
+    const int qb = static_cast<int>(gridDim.x) - 1 - static_cast<int>(blockIdx.x);  // longest first
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n32 = lane & 31, h32 = lane >> 5;
+    const int t = qb * QB + wave * 32 + n32;  // this lane's query (token index in the pass)
+    const bool live = t < p.len;
+    const int qpos = p.pos_base + min(t, p.len - 1);
+    const int last_pos = p.pos_base + min(p.len, qb * QB + QB) - 1;              // last key the workgroup needs
+    const int wave_last = p.pos_base + min(p.len, qb * QB + wave * 32 + 32) - 1;  // ... and this wavefront
+    const int wave_first = p.pos_base + min(p.len - 1, qb * QB + wave * 32);  // position of its first query
+    // Q^T as the B operand: lane (query, half) holds dims 8 c + 4 half .. + 3 for c = 0..7, pre-scaled
+    float4 qf[8];
+    {
+        const float* qr = p.q + (static_cast<size_t>(b) * p.len + min(t, p.len - 1)) * p.d_model + h * HS;
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const float4 v = *reinterpret_cast<const float4*>(qr + c * 8 + h32 * 4);
+            qf[c] = make_float4(v.x * p.scale, v.y * p.scale, v.z * p.scale, v.w * p.scale);
+        }
+    }
+    attn_v16f o[2];  // O^T: lane holds its query, dims 32 db + 8 (r / 4) + 4 half + r % 4
+#pragma unroll
+    for (int db = 0; db < 2; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+
+    // A tile on its way: 4 + 4 loads of 16 bytes per thread, rows tid / 16 + 16 r.  The
+    // cache page of a row is looked up a tile before its rows are requested, and the rows a
+    // tile before they are multiplied, so neither trip to memory is waited for in the loop;
+    // rows past the last key are read as the last key's (every query masks them).
+    attn_v4f kreg[4], vreg[4];  // native vectors: a struct copied whole into LDS keeps the array in memory
+    int page[4];
+    const int* ptab = p.kv.page_table + b * p.kv.pages_per_seq;
+    const int shift = p.kv.page_shift, slot_mask = (1 << shift) - 1;
+    const int row0 = tid >> 4, col = tid & 15;
+    const size_t kv_stride = (static_cast<size_t>(p.kv.heads) << shift) * HS;  // from a page's K rows to its V rows
+    const auto lookup = [&](int k0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) page[r] = ptab[min(k0 + row0 + 16 * r, last_pos) >> shift];
+    };
+    const auto fetch = [&](int k0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int kp = min(k0 + row0 + 16 * r, last_pos);
+            const size_t run = ((static_cast<size_t>(p.layer) * p.kv.n_pages + page[r]) * 2) * p.kv.heads + h;
+            const float* kr = p.kv.pool + ((run << shift) + (kp & slot_mask)) * HS + col * 4;
+            kreg[r] = *reinterpret_cast<const attn_v4f*>(kr);
+            vreg[r] = *reinterpret_cast<const attn_v4f*>(kr + kv_stride);
+        }
+    };
+    lookup(0);
+    fetch(0);
+    lookup(TILE);
+    for (int k0 = 0; k0 <= last_pos; k0 += TILE) {
+        __syncthreads();  // the tile before has been read by everyone
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = row0 + 16 * r;
+            *reinterpret_cast<attn_v4f*>(&Ks[row * LDK + col * 4]) = kreg[r];
+            Vt[(col * 4 + 0) * LDV + row] = vreg[r].x;
+            Vt[(col * 4 + 1) * LDV + row] = vreg[r].y;
+            Vt[(col * 4 + 2) * LDV + row] = vreg[r].z;
+            Vt[(col * 4 + 3) * LDV + row] = vreg[r].w;
+        }
+        __syncthreads();
+        fetch(k0 + TILE);  // in flight beside the products below (past the end: the last key again)
+        lookup(k0 + 2 * TILE);
+        if (k0 > wave_last) continue;  // every key of the tile is in the future of this wavefront's queries
+        // S^T: two blocks of 32 keys.  All sixteen operand reads go out before the first
+        // product: a read waited for between products leaves the matrix core idle for the
+        // LDS latency every time.  (The half of a tile on the diagonal that lies in the future
+        // of all of the wavefront's queries is multiplied too and masked: about 2 % of the
+        // products, for a loop without branches.)
+        attn_v4f ka[2][8];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int c = 0; c < 8; c++)
+                ka[kb][c] = *reinterpret_cast<const attn_v4f*>(&Ks[(kb * 32 + n32) * LDK + c * 8 + h32 * 4]);
+        __builtin_amdgcn_sched_barrier(0);
+        attn_v16f sc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) sc[kb][r] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                sc[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[kb][c][0], qf[c].x, sc[kb], 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[kb][c][1], qf[c].y, sc[kb], 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[kb][c][2], qf[c].z, sc[kb], 0, 0, 0);
+                sc[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[kb][c][3], qf[c].w, sc[kb], 0, 0, 0);
+            }
+        }
+        // the operands of the second product do not depend on the softmax: requested in front of it
+        attn_v4f va[2][2][4];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int db = 0; db < 2; db++)
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    va[kb][db][c] =
+                        *reinterpret_cast<const attn_v4f*>(&Vt[(db * 32 + n32) * LDV + kb * 32 + c * 8 + h32 * 4]);
+        __builtin_amdgcn_sched_barrier(0);
+        // causal mask (keys up to the query's own position) and the tile's maximum per query
+        float mb = -INFINITY;
+        if (k0 + TILE - 1 > wave_first) {  // only the tiles on the diagonal need the comparisons
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = k0 + kb * 32 + 8 * (r >> 2) + 4 * h32 + (r & 3);
+                    sc[kb][r] = (key <= qpos) ? sc[kb][r] : -INFINITY;
+                }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mb = fmaxf(mb, sc[kb][r]);
+        mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));  // the two halves hold different keys of the same query
+        const float mn = fmaxf(m, mb);  // finite: key 0 is never in the future
+        const float f = expf(m - mn);   // 0 on the first tile
+        float psum = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float e = expf(sc[kb][r] - mn);  // exp(-inf) = 0 for masked keys
+                sc[kb][r] = e;
+                psum += e;
+            }
+        psum += __shfl_xor(psum, 32, kWave);
+        l = l * f + psum;
+#pragma unroll
+        for (int db = 0; db < 2; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[db][r] *= f;
+        // O^T += V^T . P^T
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int db = 0; db < 2; db++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[kb][db][c][0], sc[kb][4 * c + 0], o[db], 0, 0, 0);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[kb][db][c][1], sc[kb][4 * c + 1], o[db], 0, 0, 0);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[kb][db][c][2], sc[kb][4 * c + 2], o[db], 0, 0, 0);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[kb][db][c][3], sc[kb][4 * c + 3], o[db], 0, 0, 0);
+                }
+        m = mn;
+    }
+    if (live) {
+        const float inv = 1.0f / l;
+        float* orow = p.out + (static_cast<size_t>(b) * p.len + t) * p.d_model + h * HS;
+#pragma unroll
+        for (int db = 0; db < 2; db++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++)
+                *reinterpret_cast<float4*>(orow + db * 32 + q4 * 8 + h32 * 4) =
+                    make_float4(o[db][4 * q4 + 0] * inv, o[db][4 * q4 + 1] * inv, o[db][4 * q4 + 2] * inv,
+                                o[db][4 * q4 + 3] * inv);
+    }
+}
+
 }  // namespace gh

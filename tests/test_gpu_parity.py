@@ -148,6 +148,38 @@ def test_prompt_pass_equals_steps(tiny_models, name, batch):
                         1e-6, "short prompt")
 
 
+@pytest.mark.parametrize("arch", [synth.ARCH_GPT2, synth.ARCH_MODERN])
+def test_long_prompt_pass_equals_oracle_steps(arch):
+    """Passes of 512 tokens and more run their attention 128 queries per workgroup on the
+    32 x 32 x 2 matrix product; shorter ones 64 queries per workgroup.  A 90-token pass,
+    then a 650-token pass that continues it (ragged against the 128-query blocks and the
+    64-key tiles, over scrambled 8-position pages), then a 530-token pass from an empty
+    context over the default pages: last logits and cache rows against the oracle's
+    token-by-token steps (inference.cpp:150-258)."""
+    cfg = synth.Config(arch, 211, 128, 2, 2, 760)
+    W, om = make_pair(cfg, 37, std=lively_std(cfg), norm_noise=0.1)
+    gm = G.Model.from_tensors(cfg, W)
+    batch = 2
+    toks = synth.uniform_tokens(batch * 740, cfg.vocab, 17).reshape(batch, 740)
+    a = G.Session(gm, batch=batch, shuffle_pages=True, page_tokens=8)
+    a.prefill(toks[:, :90])
+    last = a.prefill(toks[:, 90:])
+    b = G.Session(gm, batch=batch)
+    mid = b.prefill(toks[:, :530])
+    assert a.position == 740 and b.position == 530
+    for seq in range(batch):
+        osess = O.Session(om)
+        for i, t in enumerate(toks[seq]):
+            oref = osess.step(t)
+            if i == 529:
+                assert_logits_close(mid[seq], oref, TOL, f"530-token pass, arch {arch} seq {seq}")
+        assert_logits_close(last[seq], oref, TOL, f"90 + 650-token passes, arch {arch} seq {seq}")
+        for layer in range(cfg.layers):
+            for pos in (0, 89, 90, 127, 128, 601, 602, 739):
+                for kv, row in ((0, osess.k_row(layer, pos)), (1, osess.v_row(layer, pos))):
+                    assert np.abs(a.read_kv(seq, layer, kv, pos) - row).max() <= 2e-5 * max(1.0, float(np.abs(row).max()))
+
+
 def test_errors_match_the_reference(tiny_models):
     cfg, W, om, gm = tiny_models["ref-sanity-gpt2"]
     s = G.Session(gm)
