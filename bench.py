@@ -300,6 +300,9 @@ def main():
                     help="only time a two-workgroup ping-pong (same XCD / two XCDs, ordinary or device-scope "
                          "stores, non-temporal or device-scope loads, idle or beside 240 streaming workgroups) "
                          "and exit")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="only time fp32 matrix products and ordinary multiply-adds on the same SIMDs, apart and "
+                         "together (does anything issue beside a running product?), and exit")
     ap.add_argument("--phase-stamps-xcd", action="store_true",
                     help="the same for the XCD-sharded persistent kernel (eight stamps per layer)")
     a = ap.parse_args()
@@ -318,6 +321,19 @@ def main():
                     us, xa, xb = G.handoff_latency(load, store_dev, peer, busy)
                     rows.append({"busy": busy, "xcds": [xa, xb], "policy": name, "us_per_round_trip": round(us, 3)})
         print(json.dumps({"handoff": rows}))
+        return
+    if a.mfma_probe:
+        import gradhip as G
+        rows = []
+        for per in (8, 16, 24):
+            for mode, name in ((1, "products alone (wavefronts 0-3)"), (2, "multiply-adds alone (wavefronts 4-7)"),
+                               (3, "both, on the same SIMDs"), (4, "one wavefront per SIMD doing both in turn")):
+                if mode == 1 and per != 8:
+                    continue
+                prod, slot, mhz = G.mfma_issue(mode, per)
+                rows.append({"multiply_adds_per_slot": per, "what": name, "clk_per_product": round(prod, 1),
+                             "clk_per_slot": round(slot, 1), "shader_mhz": round(mhz)})
+        print(json.dumps({"mfma_issue": rows}))
         return
     if a.cache_probe:
         import gradhip as G

@@ -1725,6 +1725,62 @@ static float* scratch_on_current_device() {
     return g_scratch_ptr[dev];
 }
 
+// ---- matrix-core issue probe (gh_device_mfma_issue)
+
+// Wavefronts 0-3 of a workgroup (one per SIMD) run a dependent chain of fp32 matrix
+// products, wavefronts 4-7 (the same SIMDs) runs of VPER dependent-free multiply-adds,
+// or wavefronts 0-3 both in turn; every wavefront reports its shader-clock cycles.
+template <int VPER>
+__global__ __launch_bounds__(512) void mfma_issue_probe_kernel(long long* out, int iters, int mode, float a, float b) {
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    const int wave = threadIdx.x >> 6;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[i] = a + static_cast<float>(i);
+    __syncthreads();
+    const long long c0 = clock64(), w0 = wall_clock64();
+    if (wave < 4) {
+        if (mode & 1) {
+            for (int i = 0; i < iters; i++) {
+#pragma unroll
+                for (int u = 0; u < 8; u++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+            }
+        } else if (mode & 4) {
+            for (int i = 0; i < iters; i++) {
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < VPER; v++) x[v & 7] = x[v & 7] * b + a;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    } else if (mode & 2) {
+        for (int i = 0; i < iters; i++) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+#pragma unroll
+                for (int v = 0; v < VPER; v++) x[v & 7] = x[v & 7] * b + a;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    const long long c1 = clock64(), w1 = wall_clock64();
+    float keep = acc[0];
+#pragma unroll
+    for (int i = 0; i < 8; i++) keep += x[i];
+    if ((threadIdx.x & 63) == 0) {
+        long long* o = out + (static_cast<size_t>(blockIdx.x) * 8 + wave) * 3;
+        o[0] = c1 - c0;
+        o[1] = w1 - w0;
+        o[2] = static_cast<long long>(keep);
+    }
+}
+
 // ---- hand-off latency probe (gh_device_handoff_latency)
 
 // Workgroup 0 and workgroup `peer` bounce a counter: each waits until the other's word
@@ -2659,6 +2715,52 @@ gh_status gh_device_handoff_latency(int32_t load_policy, int32_t device_scope_st
         *us_per_round_trip = static_cast<double>(ticks[0]) / 100.0 / rounds;
         if (xcd_a) *xcd_a = static_cast<int32_t>(xcds[0]);
         if (xcd_b) *xcd_b = static_cast<int32_t>(xcds[peer]);
+    });
+}
+
+gh_status gh_device_mfma_issue(int32_t mode, int32_t valu_per_slot, double* clk_per_product, double* clk_per_valu_slot,
+                               double* shader_mhz) {
+    return guard([&] {
+        require_gpu();
+        using Kernel = void (*)(long long*, int, int, float, float);
+        Kernel kernel = valu_per_slot == 8    ? mfma_issue_probe_kernel<8>
+                        : valu_per_slot == 16 ? mfma_issue_probe_kernel<16>
+                        : valu_per_slot == 24 ? mfma_issue_probe_kernel<24>
+                                              : nullptr;
+        if (!kernel || mode < 1 || mode > 6 || (mode & 1 && mode & 4) || !clk_per_product || !clk_per_valu_slot ||
+            !shader_mhz)
+            throw ApiError{GH_ERR_INVALID_ARGUMENT, "matrix-core issue probe: mode 1, 2, 3, 4 or 6; 8, 16 or 24 "
+                                                    "multiply-adds per slot"};
+        const int blocks = 256, iters = 4000;
+        struct Scratch {
+            long long* out = nullptr;
+            ~Scratch() {
+                if (out) (void)hipFree(out);
+            }
+        } t;
+        dev_alloc(t.out, static_cast<size_t>(blocks) * 8 * 3);
+        for (int rep = 0; rep < 2; rep++) {  // the first run brings the clock up
+            hipLaunchKernelGGL(kernel, dim3(blocks), dim3(512), 0, nullptr, t.out, iters, mode, 1.0f, 0.999f);
+            HIP_CHECK(hipGetLastError());
+            HIP_CHECK(hipDeviceSynchronize());
+        }
+        std::vector<long long> h(static_cast<size_t>(blocks) * 8 * 3);
+        HIP_CHECK(hipMemcpy(h.data(), t.out, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
+        double mfma = 0.0, valu = 0.0, cyc = 0.0, wall = 0.0;
+        for (int b = 0; b < blocks; b++)
+            for (int w = 0; w < 8; w++) {
+                const long long* o = &h[(static_cast<size_t>(b) * 8 + w) * 3];
+                (w < 4 ? mfma : valu) += static_cast<double>(o[0]);
+                const bool busy = w < 4 ? (mode & 5) != 0 : (mode & 2) != 0;
+                if (busy) {
+                    cyc += static_cast<double>(o[0]);
+                    wall += static_cast<double>(o[1]);
+                }
+            }
+        const double slots = static_cast<double>(blocks) * 4 * iters * 8;
+        *clk_per_product = (mode & 5) ? mfma / slots : 0.0;
+        *clk_per_valu_slot = (mode & 2) ? valu / slots : 0.0;
+        *shader_mhz = wall > 0.0 ? cyc / wall * 100.0 : 0.0;  // the constant clock counts at 100 MHz
     });
 }
 

@@ -112,6 +112,8 @@ SYMBOLS = {
     "gh_device_reread_bandwidth": (C.c_int, [C.c_size_t, C.c_int32, C.POINTER(C.c_double)]),
     "gh_device_handoff_latency": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double),
                                             C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "gh_device_mfma_issue": (C.c_int, [C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                       C.POINTER(C.c_double)]),
 }
 
 _lib = None
@@ -170,6 +172,14 @@ def handoff_latency(load_policy: int, device_scope_store: bool, peer: int, busy:
     _check(load_library().gh_device_handoff_latency(load_policy, 1 if device_scope_store else 0, peer,
                                                     1 if busy else 0, C.byref(out), C.byref(xa), C.byref(xb)))
     return out.value, xa.value, xb.value
+
+
+def mfma_issue(mode: int, valu_per_slot: int = 8):
+    """(cycles per fp32 matrix product of wavefronts 0-3, cycles per slot of multiply-adds of
+    wavefronts 4-7, shader MHz); the modes are gh_device_mfma_issue's."""
+    a, b, c = C.c_double(0.0), C.c_double(0.0), C.c_double(0.0)
+    _check(load_library().gh_device_mfma_issue(mode, valu_per_slot, C.byref(a), C.byref(b), C.byref(c)))
+    return a.value, b.value, c.value
 
 
 def pick_noalloc(logits_ptr: int, batch: int, vocab: int, history_ptr: int, history_stride: int, n_history: int,

@@ -371,6 +371,19 @@ gh_status gh_device_reread_bandwidth(size_t bytes, int32_t passes, double* gb_pe
 gh_status gh_device_handoff_latency(int32_t load_policy, int32_t device_scope_store, int32_t peer, int32_t busy,
                                     double* us_per_round_trip, int32_t* xcd_a, int32_t* xcd_b);
 
+/* Measurement aid with no counterpart in grad.cpp: does anything else issue on a SIMD while
+ * an fp32 matrix product (v_mfma_f32_32x32x2_f32, 64 cycles) runs there?  256 workgroups of
+ * eight wavefronts, two per SIMD.  mode 1: wavefronts 0-3 run a dependent chain of products;
+ * mode 2: wavefronts 4-7 run slots of valu_per_slot (8, 16 or 24) independent multiply-adds;
+ * mode 3: both at once, on the same SIMDs; mode 4: wavefronts 0-3 alone, one slot of
+ * multiply-adds after each of their own products; mode 6: 4 and 2 together.
+ * *clk_per_product: shader-clock cycles per product of wavefronts 0-3 (per product + slot in
+ * modes 4 and 6); *clk_per_valu_slot: cycles per slot of wavefronts 4-7; *shader_mhz: the
+ * shader clock the busy wavefronts saw.  If ordinary arithmetic could run beside a product,
+ * mode 3 would cost wavefronts 4-7 what mode 2 does; on gfx950 it costs them mode 1 + mode 2. */
+gh_status gh_device_mfma_issue(int32_t mode, int32_t valu_per_slot, double* clk_per_product, double* clk_per_valu_slot,
+                               double* shader_mhz);
+
 #ifdef __cplusplus
 }
 #endif

@@ -165,3 +165,15 @@ def test_prompt_longer_than_one_pass_slice():
     nll = G.Session(gm, batch=B).score(ids, tokens[:, 1:])
     ref_nll = O.score(om, ids[7], tokens[7, 1:])
     assert np.abs(nll[7] - ref_nll).max() <= 2e-4 * max(1.0, np.abs(ref_nll).max())
+
+
+def test_matrix_core_issue_probe():
+    """gh_device_mfma_issue: a dependent chain of v_mfma_f32_32x32x2_f32 runs at one product per
+    64 cycles, and the probe refuses modes and slot sizes it has no kernel for."""
+    prod, slot, mhz = G.mfma_issue(1, 8)
+    assert 60.0 < prod < 70.0 and slot == 0.0 and 1000.0 < mhz < 3000.0
+    prod, slot, mhz = G.mfma_issue(2, 8)
+    assert prod == 0.0 and 20.0 < slot < 60.0
+    for mode, per in ((0, 8), (5, 8), (7, 8), (1, 9)):
+        with pytest.raises(Exception):
+            G.mfma_issue(mode, per)
