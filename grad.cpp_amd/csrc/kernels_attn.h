@@ -578,9 +578,10 @@ __global__ __launch_bounds__(256) void attn_prefill64_kernel(const PrefillAttnPa
 // What bounds it: on this part nothing else issues on a SIMD while an fp32 matrix product
 // runs (a wavefront's ordinary arithmetic takes as long beside another wavefront's
 // v_mfma_f32_32x32x2_f32 chain as the two take one after the other), so the softmax
-// arithmetic (about 700 vector instructions per wavefront and tile, 430 of them the 33
-// precise exponentials) adds to the 128 products of a tile instead of hiding behind them:
-// 16 x 12 heads x 1536 tokens take 0.86 ms, of which the products alone are 0.39.
+// arithmetic adds to the 128 products of a tile instead of hiding behind them.  With expf
+// it was about 700 vector instructions per wavefront and tile, 430 of them the 33
+// exponentials, and 16 x 12 heads x 1536 tokens took 0.86 ms, of which the products alone
+// are 0.39; with scores in units of ln 2 and the hardware's 2^x it is 0.78 ms.
 typedef float attn_v16f __attribute__((ext_vector_type(16)));
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill128_kernel(const PrefillAttnParams p) {
@@ -597,14 +598,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int last_pos = p.pos_base + min(p.len, qb * QB + QB) - 1;              // last key the workgroup needs
     const int wave_last = p.pos_base + min(p.len, qb * QB + wave * 32 + 32) - 1;  // ... and this wavefront
     const int wave_first = p.pos_base + min(p.len - 1, qb * QB + wave * 32);  // position of its first query
-    // Q^T as the B operand: lane (query, half) holds dims 8 c + 4 half .. + 3 for c = 0..7, pre-scaled
+    // Q^T as the B operand: lane (query, half) holds dims 8 c + 4 half .. + 3 for c = 0..7, pre-scaled.
+    // The scale carries log2(e): scores are kept in units of ln 2 and the exponentials below are the
+    // hardware's 2^x (one instruction, 1 ulp) instead of expf's thirteen.  What expf's exact argument
+    // reduction would add is below what the fp32 dot products in front of it already lose: a score s
+    // carries an error of ~|s| 2^-23 from its 64 products, and so does s log2(e) formed this way.
+    const float qscale = p.scale * 1.44269504088896341f;
     float4 qf[8];
     {
         const float* qr = p.q + (static_cast<size_t>(b) * p.len + min(t, p.len - 1)) * p.d_model + h * HS;
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             const float4 v = *reinterpret_cast<const float4*>(qr + c * 8 + h32 * 4);
-            qf[c] = make_float4(v.x * p.scale, v.y * p.scale, v.z * p.scale, v.w * p.scale);
+            qf[c] = make_float4(v.x * qscale, v.y * qscale, v.z * qscale, v.w * qscale);
         }
     }
     attn_v16f o[2];  // O^T: lane holds its query, dims 32 db + 8 (r / 4) + 4 half + r % 4
@@ -709,13 +715,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int r = 0; r < 16; r++) mb = fmaxf(mb, sc[kb][r]);
         mb = fmaxf(mb, __shfl_xor(mb, 32, kWave));  // the two halves hold different keys of the same query
         const float mn = fmaxf(m, mb);  // finite: key 0 is never in the future
-        const float f = expf(m - mn);   // 0 on the first tile
+        const float f = __builtin_amdgcn_exp2f(m - mn);  // 0 on the first tile
         float psum = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const float e = expf(sc[kb][r] - mn);  // exp(-inf) = 0 for masked keys
+                const float e = __builtin_amdgcn_exp2f(sc[kb][r] - mn);  // 2^(-inf) = 0 for masked keys
                 sc[kb][r] = e;
                 psum += e;
             }
