@@ -628,6 +628,20 @@ static int enqueue_step(Session& s, bool pick_first = false) {
     HIP_CHECK(hipGetLastError());
     launches++;
 
+    // What a projection launch touches into the L2s for the projection after it (NextWeights):
+    // the whole matrix, in the 16-row tiles that launch reads it in; at 16 sequences and fewer.
+    const bool touch = B >= kMinGemmBatch && B <= 16;
+    const auto next_matrix = [&](const float* W, int N, int K) {
+        NextWeights f{};
+        if (!touch || !gemm_shape_ok(K, K) || N % 16 != 0) return f;
+        f.base = W;
+        f.chunk_lines = K / 2;  // 16 rows of K floats
+        f.chunks = N / 16;
+        const long long lines = static_cast<long long>(f.chunks) * f.chunk_lines;
+        f.blocks = static_cast<int>(std::min<long long>(128, (lines + 8191) / 8192 * 8));  // up to four lines per thread of 256
+        return f;
+    };
+
     for (int l = 0; l < sh.layers; l++) {
         const LayerWeights& w = m.layers[l];
         GemvParams g{};
@@ -650,6 +664,7 @@ static int enqueue_step(Session& s, bool pick_first = false) {
         g.rope = modern;
         g.rope_cos = m.rope_cos;
         g.rope_sin = m.rope_sin;
+        g.next = NextWeights{};  // attention follows
         launches += modern ? project<PRO_RMSNORM, EPI_QKV>(s, g, st)
                            : project<PRO_LAYERNORM, EPI_QKV>(s, g, st);
 
@@ -677,6 +692,7 @@ static int enqueue_step(Session& s, bool pick_first = false) {
         g.in_stride = d;
         g.out = s.x;
         g.out_stride = d;
+        g.next = next_matrix(w.w1, modern ? 2 * F : F, d);
         launches += project<PRO_PLAIN, EPI_RESID>(s, g, st);
 
         // norm2 -> FFN
@@ -688,6 +704,7 @@ static int enqueue_step(Session& s, bool pick_first = false) {
         g.out_stride = F;
         g.W = w.w1;
         g.K = d;
+        g.next = next_matrix(w.w2, d, F);
         if (modern) {
             g.bias = nullptr;
             g.N = 2 * F;
@@ -705,6 +722,7 @@ static int enqueue_step(Session& s, bool pick_first = false) {
         g.in_stride = F;
         g.out = s.x;
         g.out_stride = d;
+        g.next = l + 1 < sh.layers ? next_matrix(m.layers[l + 1].wqkv, 3 * d, d) : NextWeights{};
         launches += project<PRO_PLAIN, EPI_RESID>(s, g, st);
     }
 

@@ -77,6 +77,14 @@ __global__ __launch_bounds__(64 * KW) void gemm16_kernel(const GemvParams p, int
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // id -> (weight group, row group): ids with the same id % 8 and consecutive id / 8 share weights
     const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+    {
+        // workgroups past the tiles only touch the next launch's weights into their XCD's L2
+        const int main_blocks = (((p.N + 16 * NT - 1) / (16 * NT) + 7) & ~7) * m_groups;
+        if (id >= main_blocks) {
+            touch_next_weights(p.next, id - main_blocks, 64 * KW);
+            return;
+        }
+    }
     const int n_group = xcd + 8 * (slot / m_groups), m_group = slot % m_groups;
     const int n0 = n_group * 16 * NT, m0 = m_group * 16 * MT;
     if (n0 >= p.N) return;
@@ -302,8 +310,8 @@ inline void launch_gemm16_as(const GemvParams& p, int M, hipStream_t st) {
     const int m_groups = (M + 16 * MT - 1) / (16 * MT);
     const int n_groups = (p.N + 16 * NT - 1) / (16 * NT);
     const int n_groups8 = (n_groups + 7) / 8 * 8;  // whole rounds of the 8 XCDs
-    hipLaunchKernelGGL((gemm16_kernel<EPI, RMS, MT, NT, KW>), dim3(n_groups8 * m_groups), dim3(64 * KW), 0,
-                       st, p, M, m_groups);
+    hipLaunchKernelGGL((gemm16_kernel<EPI, RMS, MT, NT, KW>), dim3(n_groups8 * m_groups + p.next.blocks),
+                       dim3(64 * KW), 0, st, p, M, m_groups);
 }
 
 // Weight tiles per workgroup of the wide kernel: 16000 rows = 250 workgroups.

@@ -15,6 +15,44 @@ namespace gh {
 enum Prologue { PRO_PLAIN = 0, PRO_LAYERNORM = 1, PRO_RMSNORM = 2 };
 enum Epilogue { EPI_STORE = 0, EPI_QKV = 1, EPI_RESID = 2, EPI_GELU = 3, EPI_SWIGLU = 4 };
 
+// What a decode launch of few rows brings into the L2s for the launch after it.  Lines
+// read by one launch are still in an XCD's L2 when the next launch on the stream reads them
+// there, and a dependent launch is little more than its start plus one trip to memory per
+// round of loads.  The next launch's matrix is cut into chunks of chunk_lines cache lines
+// (one 16-row weight tile of that launch); chunk c will be read by workgroups on XCD c % 8
+// (gemm16_kernel's id -> tile map), and `blocks` workgroups appended to the grid of this
+// launch (a multiple of 8, so workgroup b runs on XCD b % 8 like every other) read one word
+// of every line of their XCD's chunks.  It pays where the launch that carries the touches
+// is short of work anyway: 16 sequences at context 2048 0.5197 -> 0.5104 ms per step (the
+// same touches dealt to the workgroups without regard to the XCD, which only fills the
+// memory-side cache: 0.5161 -> 0.5133); at 64 sequences the carrying launches lose more
+// than the next ones gain (0.4140 -> 0.4257), so the engine asks for it at 16 rows and
+// fewer.  blocks == 0: nothing to do.
+struct NextWeights {
+    const float* base;
+    int chunk_lines;
+    int chunks;
+    int blocks;
+};
+
+// Workgroup pb of f.blocks appended ones; nthreads threads, four loads in flight each.
+__device__ __forceinline__ void touch_next_weights(const NextWeights& f, int pb, int nthreads) {
+    const int xcd = pb & 7, slot = pb >> 3, slots = f.blocks >> 3;
+    const int lines = ((f.chunks - xcd + 7) >> 3) * f.chunk_lines;  // this XCD's share
+    const int stride = slots * nthreads;
+    const int* base = reinterpret_cast<const int*>(f.base);
+    for (int i0 = slot * nthreads + static_cast<int>(threadIdx.x); i0 < lines; i0 += 4 * stride) {
+        int v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = min(i0 + u * stride, lines - 1);  // past the end: the last line again
+            const int c = xcd + 8 * (i / f.chunk_lines), l = i % f.chunk_lines;
+            v[u] = base[(static_cast<size_t>(c) * f.chunk_lines + l) * 32];
+        }
+        asm volatile("" ::"v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]));
+    }
+}
+
 struct GemvParams {
     const float* W;     // (N, K) row-major: row n holds the weights of output n
     const float* bias;  // N floats or nullptr
@@ -47,6 +85,9 @@ struct GemvParams {
     // (text_gen.cpp:52-60) without reading the row back.
     float2* best;
     int best_stride;
+    // gemm16_kernel at 16 rows and fewer: the matrix of the launch that follows this one
+    // (see NextWeights).
+    NextWeights next;
 };
 
 // What the epilogue of one pair of outputs (row, row + 1) of input row b needs
