@@ -629,8 +629,8 @@ static int enqueue_step(Session& s, bool pick_first = false) {
     launches++;
 
     // What a projection launch touches into the L2s for the projection after it (NextWeights):
-    // the whole matrix, in the 16-row tiles that launch reads it in; at 16 sequences and fewer.
-    const bool touch = B >= kMinGemmBatch && B <= 16;
+    // the whole matrix, in the 16-row tiles that launch reads it in; up to 48 sequences.
+    const bool touch = B >= kMinGemmBatch && B <= 48;
     const auto next_matrix = [&](const float* W, int N, int K) {
         NextWeights f{};
         if (!touch || !gemm_shape_ok(K, K) || N % 16 != 0) return f;

@@ -15,19 +15,20 @@ namespace gh {
 enum Prologue { PRO_PLAIN = 0, PRO_LAYERNORM = 1, PRO_RMSNORM = 2 };
 enum Epilogue { EPI_STORE = 0, EPI_QKV = 1, EPI_RESID = 2, EPI_GELU = 3, EPI_SWIGLU = 4 };
 
-// What a decode launch of few rows brings into the L2s for the launch after it.  Lines
+// What a decode launch of a few dozen rows brings into the L2s for the launch after it.  Lines
 // read by one launch are still in an XCD's L2 when the next launch on the stream reads them
 // there, and a dependent launch is little more than its start plus one trip to memory per
 // round of loads.  The next launch's matrix is cut into chunks of chunk_lines cache lines
 // (one 16-row weight tile of that launch); chunk c will be read by workgroups on XCD c % 8
 // (gemm16_kernel's id -> tile map), and `blocks` workgroups appended to the grid of this
 // launch (a multiple of 8, so workgroup b runs on XCD b % 8 like every other) read one word
-// of every line of their XCD's chunks.  It pays where the launch that carries the touches
-// is short of work anyway: 16 sequences at context 2048 0.5197 -> 0.5104 ms per step (the
-// same touches dealt to the workgroups without regard to the XCD, which only fills the
-// memory-side cache: 0.5161 -> 0.5133); at 64 sequences the carrying launches lose more
-// than the next ones gain (0.4140 -> 0.4257), so the engine asks for it at 16 rows and
-// fewer.  blocks == 0: nothing to do.
+// of every line of their XCD's chunks.  Per decode step of the 69M Llama block at context
+// 256, without and with: 2 sequences 247.0 -> 243.4 us, 8: 252.3 -> 248.2, 16: 277.3 ->
+// 268.3, 24: 312.0 -> 299.7, 32: 328.6 -> 310.7, 48: 377.4 -> 371.2, 64: 397.6 -> 409.0; 16
+// sequences at context 2048 516.0 -> 509.5 (the same touches dealt to the workgroups
+// without regard to the XCD, which only fills the memory-side cache: 516.1 -> 513.3).  At 64
+// sequences the launches that carry the touches lose more than the next ones gain, so the
+// engine asks for it up to 48.  blocks == 0: nothing to do.
 struct NextWeights {
     const float* base;
     int chunk_lines;
@@ -85,7 +86,7 @@ struct GemvParams {
     // (text_gen.cpp:52-60) without reading the row back.
     float2* best;
     int best_stride;
-    // gemm16_kernel at 16 rows and fewer: the matrix of the launch that follows this one
+    // gemm16_kernel up to 48 rows: the matrix of the launch that follows this one
     // (see NextWeights).
     NextWeights next;
 };
