@@ -1,11 +1,12 @@
 """gh_pick_noalloc, the entry point that allocates nothing: its picks must be those of
-gh_session_pick on the same logits, history, options and draws, on two calls in a row,
+gh_session_pick, and of the CPU checker, on the same logits, history, options and draws, on two calls in a row,
 the second with a smaller input (the shared working rows keep the first call's
 contents).  Device memory for the caller's side comes from torch."""
 import numpy as np
 import pytest
 
 import gradhip as G
+import oracle_lib as O
 from gradhip import synth
 
 pytestmark = pytest.mark.gpu
@@ -40,6 +41,19 @@ def _case(torch, cfg, seed, batch, plen):
     logits = gs.prefill(prompts)
     u = synth.uniforms(batch, seed + 2)
     want = [gs.pick(G.sampling(**o), uniforms=u).copy() for o in OPTIONS]
+    # ... which are the CPU checker's own from the same logits, history and draws (text_gen.cpp:14-33,
+    # :52-60, :135-209): the comparison below is with the reference's arithmetic, not only with the session's
+    # (not the top-p walk over a whole vocabulary of 50 k nearly equal probabilities: there the rounding
+    # of the running sum decides between neighbours, which the sampler's own tests hold to the checker
+    # with their near-tie rule)
+    for o, picks in zip(OPTIONS, want):
+        if not o.get("greedy") and o.get("top_k", 0) == 0 and cfg.vocab > 10000:
+            continue
+        for b in range(batch):
+            row = O.logits_with_penalty(logits[b], prompts[b], o.get("repetition_penalty", 1.0))
+            ref = O.argmax_first(row) if o.get("greedy") else O.sample_from_logits(
+                row, o.get("temperature", 1.0), o.get("top_k", 0), o.get("top_p", 1.0), float(u[b]))
+            assert int(picks[b]) == int(ref), (o, b, int(picks[b]), int(ref))
     dev = dict(logits=torch.from_numpy(np.ascontiguousarray(logits)).cuda(),
                hist=torch.from_numpy(np.ascontiguousarray(prompts.astype(np.int32))).cuda(),
                u=torch.from_numpy(u.astype(np.float32)).cuda(),
