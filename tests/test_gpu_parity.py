@@ -66,7 +66,7 @@ def test_page_size_and_placement_do_not_change_results(tiny_models):
         assert np.array_equal(ref, out)
 
 
-@pytest.mark.parametrize("batch", [2, 5, 17, 64])
+@pytest.mark.parametrize("batch", [2, 5, 17, 40, 64])
 @pytest.mark.parametrize("name", ["hs64-gpt2", "hs64-modern", "d256-modern", "odd-gpt2", "ref-metal-modern"])
 def test_batched_step_equals_per_sequence_oracle(tiny_models, name, batch):
     cfg, W, om, gm = tiny_models[name]
