@@ -1218,7 +1218,15 @@ static std::unique_ptr<Session> create_session(const Model& m, const gh_session_
             const size_t work = d + std::max(d, F) + 192 + kPersistWaves * 4 * 68 + s.pages_per_seq;
             const size_t pick = (s.pick_row_in_lds ? V : 0) + kPickWorkFloats;
             s.persist_lds = std::max(work, pick) * sizeof(float);
-            s.persist_grid = std::min(prop.multiProcessorCount, 256);
+            // As many workgroups as give every wavefront exactly one item of the widest phase (the
+            // FFN1 row pairs): workgroups beyond that have nothing to do there and still take part
+            // in every exchange.  Per token: d512 F2048 (GPT-2) 75.2 us on 256 workgroups, 67.4 on
+            // 128; d768 F3072 (GPT-2) 127.0 on 256, 119.0 on 192; the Llama block d768 F2048 (2048
+            // items) 116.9 on 256, 129.5 on 192.  Between these sizes every step of 16 either way
+            // is slower.
+            const int ffn1_items = static_cast<int>(sh.modern() ? F : F / 2);
+            const int want = ((ffn1_items + kPersistWaves - 1) / kPersistWaves + 15) / 16 * 16;
+            s.persist_grid = std::min(std::min(prop.multiProcessorCount, 256), std::max(32, want));
             // the exchange cells, the token cell (and one of padding), then what the workgroups
             // leave for a pick each of them makes itself: nine planes of one cell per
             // workgroup and a stop word

@@ -647,8 +647,9 @@ __global__ __launch_bounds__(kPersistThreads) void persist_decode_kernel(const P
             // further on, which are idle in this phase.  They need q only, leave (maximum, sum,
             // 64 weighted sums) in cells, and the head's workgroup folds the shares in a fixed order.
             const int ctx = pos + 1;
+            // (no more shares than the grid has groups of 16 workgroups: the head's own and G / 16 - 1 others)
             const int n_shares =
-                ctx <= kAttnShareFrom ? 1 : min(kAttnMaxShares, (ctx + kAttnShare - 1) / kAttnShare);  // uniform
+                ctx <= kAttnShareFrom ? 1 : min(min(kAttnMaxShares, G >> 4), (ctx + kAttnShare - 1) / kAttnShare);  // uniform
             const bool head_wg = wg < H;
             const bool share_wg = !head_wg && (wg & 15) < H && (wg >> 4) < n_shares;
             if (head_wg || share_wg) {

@@ -129,6 +129,8 @@ def test_long_context_runs_of_more_than_64_positions_per_wavefront():
     (synth.ARCH_MODERN, 768, 12, 1800, 1480),  # 6, 7, 8 shares
     (synth.ARCH_GPT2, 1024, 16, 640, 470),     # every workgroup of the first 16 has a head; 1 share, then 3
     (synth.ARCH_MODERN, 768, 12, 4096, 3800),  # 15, then 16 shares: the largest context
+    (synth.ARCH_GPT2, 512, 8, 2400, 2230),     # a grid of 128 workgroups has 8 groups of 16: 9, then 10 shares asked for, 8 made
+    (synth.ARCH_GPT2, 768, 12, 3400, 3260),    # a grid of 192: 13, then 14 shares asked for, 12 made
 ])
 def test_long_context_shared_by_several_workgroups(arch, d, heads, max_len, start):
     """Beyond 512 positions the context of a head is cut into shares of at most 256 positions: the
